@@ -51,7 +51,7 @@ def _load_builtin() -> None:
     global _BUILTIN_LOADED
     if not _BUILTIN_LOADED:
         _BUILTIN_LOADED = True
-        from ..engine import llama  # noqa: F401
+        from ..engine import begopel, llama  # noqa: F401
 
 
 _OUTSIDE_LOADED = False
@@ -89,12 +89,12 @@ def known_architectures() -> list[str]:
 
 
 def architecture_name(config_dict: dict) -> str:
-    archs = config_dict.get("architectures")
+    archs = config_dict.get("architectures") or config_dict.get("architecture")     # a list, or one name under either key
     if isinstance(archs, (list, tuple)) and archs:
         return str(archs[0])
     if isinstance(archs, str):
         return archs
-    raise ConfigError("architectures: missing; config.json must name its architecture "
+    raise ConfigError("architectures: missing; config.json must name its architecture (`architectures` or `architecture`) "
                       f"(known: {', '.join(known_architectures())})")
 
 

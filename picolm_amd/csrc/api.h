@@ -34,6 +34,9 @@ int picolm_mfma_probe(void* sink, int blocks, int iters, int random_operands, hi
 
 int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
                  int V, hipStream_t stream);
+// x[t] = table[tokens[t]] * scale, the product taken in float
+int picolm_embed_scaled(const void* table, int table_dt, const int32_t* tokens, float* x, int T, int D,
+                        int V, float scale, hipStream_t stream);
 int picolm_gather_i32(int32_t* out, const int32_t* src, const int32_t* index, int n, hipStream_t stream);   // out[i] = src[index[i]]
 int picolm_rmsnorm(const float* x, const float* w, void* out, int out_dt, const int32_t* rows,
                    int n_rows, int D, float eps, hipStream_t stream);
@@ -105,6 +108,31 @@ int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, void* C, int
 // kernels' operands.
 // Fills k_idx[key * d + i] and v_idx[i * 64 + key] with the offsets of K[key][i] and V^T[i][key].
 int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
+// What the vector-ALU attention kernels take beside keys, values and a scale (all optional: zero
+// or null is "none"): values of a size of their own, a bias by distance added to the scaled score
+// (bias[min(n, bias_rows - 1)][head] for a key n positions back), a sink (exp(sink[head]) joins the
+// softmax's denominator once, with no key and no value), and a gate (the output of head h is
+// multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows).
+typedef struct {
+    int32_t v_head_dim;
+    const float* bias;
+    int32_t bias_rows;
+    const float* sink;
+    const float* gate;
+    int32_t gate_stride;
+} picolm_attn_extras;
+// picolm_attn_prefill_generic / picolm_attn_decode_generic over pages kept as plain arrays K[64][d],
+// V^T[dv][64] whatever the dtype and head size, with the extras above; out rows are [H][dv] and the
+// partial results [n_seq][H][max_splits][dv + 2].
+int picolm_attn_prefill_plain(const void* q, const void* k_pages, const void* v_pages, void* out, int dt, const int32_t* tile_seq,
+                              const int32_t* tile_q0, int n_tiles, const int32_t* seq_slot, const int32_t* seq_pos0,
+                              const int32_t* seq_nnew, const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                              int ring_pages, int H, int G, int d, int window, float scale, const picolm_attn_extras* x,
+                              hipStream_t stream);
+int picolm_attn_decode_plain(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int dt, int n_seq,
+                             const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
+                             const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
+                             const picolm_attn_extras* x, hipStream_t stream);
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

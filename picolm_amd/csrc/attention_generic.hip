@@ -27,7 +27,8 @@ template <typename T, int MAXD>
 __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     extern __shared__ float lds[];
     const int d = a.d;
-    const int dl = min(d, AT_CHUNK), dp = dl + 1;
+    const int dv = a.dv > 0 ? a.dv : d;         // a value's size
+    const int dl = min(d, AT_CHUNK), dp = min(max(d, dv), AT_CHUNK) + 1;
     const bool whole = d <= AT_CHUNK;           // the queries lie in LDS once and for all
     float* Qs = lds;                            // [AT_ROWS][dl]
     float* KVs = Qs + AT_ROWS * dl;             // [PAGE][dl+1]
@@ -96,18 +97,19 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     }
     // PV ownership: thread -> (row pr, column group pc), columns pc + 16*j
     const int pr = tid / 16, pc = tid % 16;
-    const int n_cg = pc < d ? (d - pc + 15) / 16 : 0;      // this thread's columns pc + 16*j below d
+    const int n_cg = pc < dv ? (dv - pc + 15) / 16 : 0;    // this thread's columns pc + 16*j below dv
     float acc[MAXD / 16];
 #pragma unroll
     for (int j = 0; j < MAXD / 16; ++j) acc[j] = 0.f;
 
     const int slot = a.decode ? work.slot : a.seq_slot[seq];
     const int32_t* pt = a.page_table + (size_t)slot * a.max_pages;
-    const size_t page_elems = (size_t)a.G * PAGE_TOKENS * d;
+    const size_t page_elems = (size_t)a.G * PAGE_TOKENS * d, v_page_elems = (size_t)a.G * PAGE_TOKENS * dv;
 
     for (int page = page_lo; page < page_hi; ++page) {
         const int phys = pt[page % a.ring_pages];
         const size_t base = (size_t)phys * page_elems + (size_t)g * PAGE_TOKENS * d;
+        const size_t v_base = (size_t)phys * v_page_elems + (size_t)g * PAGE_TOKENS * dv;
         const int key0 = page * PAGE_TOKENS;
         const int n_keys = min(PAGE_TOKENS, hi - key0 + 1);   // rows beyond are not this sequence's
         // scores: wave handles rows 4*wave .. +3, lane = key; a head wider than the chunk adds up piece by piece
@@ -137,7 +139,11 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
                 const int r = 4 * wave + i;
                 const int qp = row_qpos[r];
                 const bool vis = r < n_rows && kpos <= qp && (a.window <= 0 || qp - kpos < a.window);
-                const float sc = vis ? s[i] * a.scale : NEG_BIG;
+                float sc = NEG_BIG;
+                if (vis) {
+                    sc = s[i] * a.scale;
+                    if (a.bias) sc += a.bias[(size_t)min(qp - kpos, a.bias_rows - 1) * a.H + row_head[r]];
+                }
                 const float m_new = fmaxf(m_run[i], wave_max(sc));
                 const float p = vis ? expf(sc - m_new) : 0.f;
                 const float al = expf(m_run[i] - m_new);
@@ -154,10 +160,10 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
         for (int ci = 0; ci < MAXD / AT_CHUNK; ++ci) {
             const int c0 = ci * AT_CHUNK;
-            if (c0 >= d) break;
-            const int dc = min(AT_CHUNK, d - c0);
+            if (c0 >= dv) break;
+            const int dc = min(AT_CHUNK, dv - c0);
             if (ci > 0) __syncthreads();                       // the piece before has been used
-            const T* vp = (const T*)a.v_pages + base + (size_t)c0 * PAGE_TOKENS;       // transposed: [d][PAGE]
+            const T* vp = (const T*)a.v_pages + v_base + (size_t)c0 * PAGE_TOKENS;     // transposed: [dv][PAGE]
             for (int idx = tid; idx < PAGE_TOKENS * dc; idx += AT_THREADS) {
                 const int c = idx / PAGE_TOKENS, r = idx % PAGE_TOKENS;
                 KVs[r * dp + c] = r < n_keys ? to_f32<T>(vp[idx]) : 0.f;
@@ -185,7 +191,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
     if (pr >= n_rows) return;
     const int tok = row_tok[pr], head = row_head[pr];
     if (a.decode && work.n_chunks > 1) {
-        float* po = a.partial + (((size_t)seq * a.H + head) * a.max_splits + split) * (d + 2);
+        float* po = a.partial + (((size_t)seq * a.H + head) * a.max_splits + split) * (dv + 2);
         if (pc == 0) {
             po[0] = m_s[pr];
             po[1] = l_s[pr];
@@ -194,12 +200,22 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
         for (int j = 0; j < MAXD / 16; ++j)
             if (j < n_cg) po[2 + pc + 16 * j] = acc[j];
     } else {
-        const float l = l_s[pr];
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        T* o = (T*)a.out + (size_t)tok * a.H * d + (size_t)head * d;
+        float l = l_s[pr], keep = 1.f;
+        if (a.sink) {                   // one more term of the denominator, under a maximum that covers it
+            const float m = m_s[pr], top = fmaxf(m, a.sink[head]);
+            keep = expf(m - top);
+            l = l * keep + expf(a.sink[head] - top);
+        }
+        const float inv = l > 0.f ? keep / l : 0.f;
+        T* o = (T*)a.out + (size_t)tok * a.H * dv + (size_t)head * dv;
+        const float* gate = a.gate ? a.gate + (size_t)tok * a.gate_stride + (size_t)head * dv : nullptr;
 #pragma unroll
         for (int j = 0; j < MAXD / 16; ++j)
-            if (j < n_cg) o[pc + 16 * j] = from_f32<T>(acc[j] * inv);
+            if (j < n_cg) {
+                float y = acc[j] * inv;
+                if (gate) y *= 1.f / (1.f + expf(-gate[pc + 16 * j]));
+                o[pc + 16 * j] = from_f32<T>(y);
+            }
     }
 }
 
@@ -211,7 +227,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
     const int unit = blockIdx.x * MERGE_WAVES + threadIdx.x / WAVE;
     const int lane = threadIdx.x % WAVE;
     if (unit >= n_units) return;
-    const int H = a.H, d = a.d;
+    const int H = a.H, d = a.dv > 0 ? a.dv : a.d;        // columns of a value
     const int seq = unit / H, head = unit % H;
     const int qpos = a.seq_pos0[seq];
     const int n_splits = (qpos / 64 + 1 - decode_first_page(a.window, qpos) + a.pages_per_chunk - 1) / a.pages_per_chunk;
@@ -231,12 +247,15 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
         }
     float m = NEG_BIG;
     for (int i = lane; i < n_splits; i += WAVE) m = fmaxf(m, p[(size_t)i * stride]);
-    const float M = wave_max(m);
+    float M = wave_max(m);
+    if (a.sink) M = fmaxf(M, a.sink[head]);
     float l = 0.f;
     for (int i = lane; i < n_splits; i += WAVE) l += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 1];
-    const float L = wave_sum(l);
+    float L = wave_sum(l);
+    if (a.sink) L += expf(a.sink[head] - M);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     T* o = (T*)a.out + (size_t)seq * H * d + (size_t)head * d;
+    const float* gate = a.gate ? a.gate + (size_t)seq * a.gate_stride + (size_t)head * d : nullptr;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int c = lane + j * WAVE;
@@ -246,23 +265,25 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(AttnArgs
         for (int i = 0; i < EARLY; ++i)
             if (i < n_splits) acc += expf(p[(size_t)i * stride] - M) * early[i][j];
         for (int i = EARLY; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
+        if (gate) acc *= 1.f / (1.f + expf(-gate[c]));
         o[c] = from_f32<T>(acc * inv);
     }
     for (int c = lane + 4 * WAVE; c < d; c += WAVE) {       // a head wider than 256
         float acc = 0.f;
         for (int i = 0; i < n_splits; ++i) acc += expf(p[(size_t)i * stride] - M) * p[(size_t)i * stride + 2 + c];
+        if (gate) acc *= 1.f / (1.f + expf(-gate[c]));
         o[c] = from_f32<T>(acc * inv);
     }
 }
 
-static size_t attn_lds_bytes(int d) {
-    const int dl = d < AT_CHUNK ? d : AT_CHUNK;
-    return sizeof(float) * ((size_t)AT_ROWS * dl + (size_t)PAGE_TOKENS * (dl + 1) + AT_ROWS * PAGE_TOKENS + 3 * AT_ROWS);
+static size_t attn_lds_bytes(int d, int dv) {
+    const int dl = d < AT_CHUNK ? d : AT_CHUNK, widest = d > dv ? d : dv, dp = (widest < AT_CHUNK ? widest : AT_CHUNK) + 1;
+    return sizeof(float) * ((size_t)AT_ROWS * dl + (size_t)PAGE_TOKENS * dp + AT_ROWS * PAGE_TOKENS + 3 * AT_ROWS);
 }
 
 template <typename T, int MAXD>
 static int launch_attn_sized(const AttnArgs& a, dim3 grid, hipStream_t stream) {
-    const size_t lds = attn_lds_bytes(a.d);
+    const size_t lds = attn_lds_bytes(a.d, a.dv > 0 ? a.dv : a.d);
     static size_t raised = 48 * 1024;      // what a kernel may use without asking
     if (lds > raised) {
         hipError_t e = hipFuncSetAttribute((const void*)attn_tile_kernel<T, MAXD>,
@@ -279,7 +300,8 @@ static int launch_attn_sized(const AttnArgs& a, dim3 grid, hipStream_t stream) {
 // (heads of up to 256 have the kernel with 16 accumulators a thread, wider ones that with 64)
 template <typename T>
 static int launch_attn(const AttnArgs& a, dim3 grid, hipStream_t stream) {
-    return a.d <= AT_CHUNK ? launch_attn_sized<T, AT_CHUNK>(a, grid, stream) : launch_attn_sized<T, AT_MAX_D>(a, grid, stream);
+    return a.d <= AT_CHUNK && a.dv <= AT_CHUNK ? launch_attn_sized<T, AT_CHUNK>(a, grid, stream)
+                                               : launch_attn_sized<T, AT_MAX_D>(a, grid, stream);
 }
 
 int check_decode_chunks(const char* who, const float* partial, const int32_t* chunk_list, int n_chunks,
@@ -348,6 +370,68 @@ extern "C" int picolm_attn_decode_generic(const void* q, const void* k_pages, co
     AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
                   page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
                   nullptr, nullptr, nullptr, nullptr, 0};
+    dim3 grid(n_chunks * G * chunks);
+    const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
+    if (rc) return rc;
+    return max_splits > 1 ? picolm_attn_merge_launch(a, dt, n_seq, stream) : 0;
+}
+
+// The same kernels for a caller that keeps its pages as plain arrays whatever the dtype and head
+// size (a called operation that writes its own pages), with what `x` adds: values of another size
+// than keys, a bias by distance, a sink in the softmax's denominator, a gate on the output.
+static void with_extras(AttnArgs& a, const picolm_attn_extras* x) {
+    if (!x) return;
+    a.dv = x->v_head_dim == a.d ? 0 : x->v_head_dim;
+    a.bias = x->bias;
+    a.bias_rows = x->bias_rows;
+    a.sink = x->sink;
+    a.gate = x->gate;
+    a.gate_stride = x->gate_stride;
+}
+
+static int check_extras(const char* who, const picolm_attn_extras* x, int H, int d) {
+    if (!x) return 0;
+    PICOLM_REQUIRE(x->v_head_dim >= 0 && x->v_head_dim <= AT_MAX_D, "%s: value size %d is not in [1, %d]", who, x->v_head_dim, AT_MAX_D);
+    PICOLM_REQUIRE(!x->bias || x->bias_rows >= 1, "%s: a bias by distance needs at least one row", who);
+    const int dv = x->v_head_dim > 0 ? x->v_head_dim : d;
+    PICOLM_REQUIRE(!x->gate || x->gate_stride >= H * dv, "%s: gate rows of %d floats for %d heads of %d", who, x->gate_stride, H, dv);
+    return 0;
+}
+
+extern "C" int picolm_attn_prefill_plain(const void* q, const void* k_pages, const void* v_pages, void* out, int dt,
+                                         const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles, const int32_t* seq_slot,
+                                         const int32_t* seq_pos0, const int32_t* seq_nnew, const int32_t* cu_seqlens,
+                                         const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window,
+                                         float scale, const picolm_attn_extras* x, hipStream_t stream) {
+    if (check_attn_sizes("attn_prefill_plain", H, G, d, max_pages, ring_pages)) return -1;
+    if (check_extras("attn_prefill_plain", x, H, d)) return -1;
+    PICOLM_REQUIRE(H <= 65535, "attn_prefill_plain: %d heads exceed the grid", H);
+    PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_prefill_plain: unknown dtype %d", dt);
+    if (n_tiles <= 0) return 0;
+    AttnArgs a = {q, k_pages, v_pages, out, nullptr, tile_seq, tile_q0, seq_slot, seq_pos0, seq_nnew,
+                  cu_seqlens, page_table, max_pages, ring_pages, H, G, d, window, scale, 0, nullptr, 0, 1,
+                  nullptr, nullptr, nullptr, nullptr, 0};
+    with_extras(a, x);
+    dim3 grid(n_tiles, H);
+    return dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
+}
+
+extern "C" int picolm_attn_decode_plain(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int dt,
+                                        int n_seq, const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits,
+                                        const int32_t* seq_pos0, const int32_t* page_table, int max_pages, int ring_pages, int H, int G,
+                                        int d, int window, float scale, const picolm_attn_extras* x, hipStream_t stream) {
+    if (check_attn_sizes("attn_decode_plain", H, G, d, max_pages, ring_pages)) return -1;
+    if (check_extras("attn_decode_plain", x, H, d)) return -1;
+    if (check_decode_chunks("attn_decode_plain", partial, chunk_list, n_chunks, pages_per_chunk, max_splits)) return -1;
+    PICOLM_REQUIRE(dt == PICOLM_F32 || dt == PICOLM_BF16, "attn_decode_plain: unknown dtype %d", dt);
+    if (n_seq <= 0 || n_chunks <= 0) return 0;
+    const int chunks = ceil_div(H / G, AT_ROWS);
+    PICOLM_REQUIRE((int64_t)n_chunks * G * chunks < (1ll << 31), "attn_decode_plain: %d chunks of %d workgroups exceed the grid", n_chunks,
+                   G * chunks);
+    AttnArgs a = {q, k_pages, v_pages, out, partial, nullptr, nullptr, nullptr, seq_pos0, nullptr, nullptr,
+                  page_table, max_pages, ring_pages, H, G, d, window, scale, 1, chunk_list, pages_per_chunk, max_splits,
+                  nullptr, nullptr, nullptr, nullptr, 0};
+    with_extras(a, x);
     dim3 grid(n_chunks * G * chunks);
     const int rc = dt == PICOLM_F32 ? launch_attn<float>(a, grid, stream) : launch_attn<bf16_t>(a, grid, stream);
     if (rc) return rc;

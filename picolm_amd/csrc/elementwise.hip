@@ -5,16 +5,17 @@
 #include "attention.h"
 
 // ---- embedding: x[t][:] = table[tokens[t]][:] ------------------------------------------
-// picolm/model_core.c:1785-1786, :2758-2762: the row is converted to float, no scaling.
+// picolm/model_core.c:1785-1786, :2758-2762: the row is converted to float, no scaling; a model
+// that scales its embedding says by how much (the product is taken in float).
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int32_t* __restrict__ tokens,
-                             float* __restrict__ x, int D, int V) {
+                             float* __restrict__ x, int D, int V, float scale) {
     const int t = blockIdx.x;
     int tok = tokens[t];
     tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);      // ids are checked on the host; stay in bounds anyway
     const TW* row = table + (size_t)tok * D;
     float* out = x + (size_t)t * D;
-    for (int i = threadIdx.x; i < D; i += blockDim.x) out[i] = to_f32<TW>(row[i]);
+    for (int i = threadIdx.x; i < D; i += blockDim.x) out[i] = to_f32<TW>(row[i]) * scale;
 }
 
 // out[i] = src[index[i]]: the tokens of the sequences that go on, picked from what a sampling kernel
@@ -34,13 +35,18 @@ extern "C" int picolm_gather_i32(int32_t* out, const int32_t* src, const int32_t
 
 extern "C" int picolm_embed(const void* table, int table_dt, const int32_t* tokens, float* x,
                             int T, int D, int V, hipStream_t stream) {
+    return picolm_embed_scaled(table, table_dt, tokens, x, T, D, V, 1.f, stream);
+}
+
+extern "C" int picolm_embed_scaled(const void* table, int table_dt, const int32_t* tokens, float* x,
+                                   int T, int D, int V, float scale, hipStream_t stream) {
     PICOLM_REQUIRE(T >= 0 && D > 0 && V > 0, "embed: bad sizes T=%d D=%d V=%d", T, D, V);
     if (T == 0) return 0;
     dim3 grid(T), block(256);
     if (table_dt == PICOLM_F32)
-        embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, tokens, x, D, V);
+        embed_kernel<float><<<grid, block, 0, stream>>>((const float*)table, tokens, x, D, V, scale);
     else if (table_dt == PICOLM_BF16)
-        embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, tokens, x, D, V);
+        embed_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)table, tokens, x, D, V, scale);
     else
         PICOLM_REQUIRE(false, "embed: unknown table dtype %d", table_dt);
     PICOLM_LAUNCH_CHECK("embed");

@@ -101,6 +101,7 @@ typedef int (*picolm_call_fn)(void* user, const picolm_step_view* view);
 // One operation.  Buffers are indices into the program's buffers.  Fields an operation does not
 // use are zero.
 //   EMBED      out[t] = weight[tokens[t]] widened to float          weight [n][k] of weight_dt
+//              scale != 0: times scale
 //   RMSNORM    out = in / sqrt(mean(in^2) + eps) * weight           weight float [k]; in float
 //   LINEAR     out (=, +=, = silu-gated) in weight^T                weight [n][k]; epilogue 0, 1, 2
 //              in_norm_weight: `in` is scratch and the input is rmsnorm(in_norm_x) with that weight

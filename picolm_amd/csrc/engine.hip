@@ -1297,7 +1297,8 @@ static int run_program(picolm_engine* e, const StepPlan& p, Workspace& w, hipStr
         if (e->timing()) TRY(timing_event(e, &before, stream));
         switch (o.kind) {
             case PICOLM_OP_EMBED:
-                TRY(picolm_embed(o.weight, o.weight_dt, p.at(p.tokens), (float*)r.buf(o.out), p.T, o.k, o.n, stream));
+                TRY(picolm_embed_scaled(o.weight, o.weight_dt, p.at(p.tokens), (float*)r.buf(o.out), p.T, o.k, o.n,
+                                        o.scale != 0.f ? o.scale : 1.f, stream));
                 break;
             case PICOLM_OP_RMSNORM: {
                 r.prepared = Prepared();

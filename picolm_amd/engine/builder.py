@@ -6,7 +6,7 @@ import torch
 from ..config import read_config_json, resolve
 from ..parts.base import Runtime
 from ..weights import Checkpoint, RandomWeights
-from . import llama as _llama  # noqa: F401  (registers the architecture)
+from . import begopel as _begopel, llama as _llama  # noqa: F401  (register the architectures)
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
            "fp32": torch.float32}

@@ -108,7 +108,7 @@ class DecoderModel:
         for spec in self.tensor_specs():
             n = 1
             for d in spec.shape:
-                n *= int(d)
+                n *= max(int(d), 0)
             total += n * size
         return total
 

@@ -156,9 +156,10 @@ class ProgramBuilder:
         self.keep.append(t)
         return t.data_ptr()
 
-    def embed(self, table: torch.Tensor, out: int) -> None:
+    def embed(self, table: torch.Tensor, out: int, scale: float = 1.0) -> None:
+        """out[t] = table[tokens[t]] widened to float, times `scale`."""
         self.ops.append(Op(kind=OP_EMBED, rows=ROWS_STEP, out=out, weight=self._ptr(table), weight_dt=_DT[table.dtype],
-                           n=table.shape[0], k=table.shape[1]))
+                           n=table.shape[0], k=table.shape[1], scale=0.0 if scale == 1.0 else float(scale)))
 
     def rmsnorm(self, norm: NormRef, x: int, out: int, rows: int = ROWS_STEP) -> None:
         self.ops.append(Op(kind=OP_RMSNORM, rows=rows, inp=x, out=out, weight=self._ptr(norm.weight), k=norm.weight.shape[0],

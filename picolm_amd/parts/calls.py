@@ -1,0 +1,58 @@
+"""The library's called operations (csrc/mixers.h) as a part emits them: each is a C function that
+the engine hands the running step to, with a structure of sizes, offsets, constants and device
+pointers.  The structures here mirror that header field by field."""
+from __future__ import annotations
+
+from ctypes import Structure, c_float, c_int32, c_int64, c_void_p
+
+from .. import kernels
+
+
+class LoopInputArgs(Structure):
+    _fields_ = [("step", c_void_p), ("width", c_int32)]
+
+
+class SinkAttentionArgs(Structure):
+    _fields_ = [("n_heads", c_int32), ("n_kv_heads", c_int32), ("head_dim", c_int32), ("v_head_dim", c_int32),
+                ("in_stride", c_int32), ("q_off", c_int32), ("k_off", c_int32), ("v_off", c_int32), ("gate_off", c_int32),
+                ("scale", c_float), ("eps", c_float),
+                ("q_norm", c_void_p), ("k_norm", c_void_p), ("bias", c_void_p), ("bias_rows", c_int32), ("sink", c_void_p)]
+
+
+class ShortConvArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("bias", c_void_p), ("channels", c_int32), ("taps", c_int32),
+                ("in_stride", c_int32), ("in_off", c_int32), ("out_stride", c_int32), ("out_off", c_int32),
+                ("state_off", c_int64), ("act", c_int32)]
+
+
+class StateScanArgs(Structure):
+    _fields_ = [("rule", c_int32), ("n_heads", c_int32), ("n_key_heads", c_int32), ("key_dim", c_int32), ("value_dim", c_int32),
+                ("in_stride", c_int32), ("a_off", c_int32), ("w_off", c_int32),
+                ("qkv_stride", c_int32), ("q_off", c_int32), ("k_off", c_int32), ("v_off", c_int32),
+                ("A_log", c_void_p), ("dt_bias", c_void_p), ("skip", c_void_p),
+                ("unit_qk", c_int32), ("unit_eps", c_float), ("q_scale", c_float), ("state_off", c_int64)]
+
+
+class GatedNormArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("weight_len", c_int32), ("width", c_int32), ("group", c_int32), ("eps", c_float),
+                ("gate_first", c_int32), ("gate_stride", c_int32), ("gate_off", c_int32)]
+
+
+class NormedSumArgs(Structure):
+    _fields_ = [("w_a", c_void_p), ("w_b", c_void_p), ("width", c_int32), ("eps", c_float), ("mult", c_float)]
+
+
+class MapRowsArgs(Structure):
+    _fields_ = [("kind", c_int32), ("width", c_int32), ("in_dtype", c_int32), ("out_dtype", c_int32), ("param", c_float)]
+
+
+MAP_RELU_SQUARED, MAP_SOFTCAP = 1, 2
+RULE_OUTER_PRODUCT, RULE_DELTA = 0, 1
+STATE_SCAN_MAX_KEY_DIM = 256
+SHORT_CONV_MAX_TAPS = 16
+
+
+def emit_library_call(b, name: str, args: Structure, out: int, **kw) -> None:
+    """Appends the library's operation `name` (`picolm_call_<name>`) with its arguments to the
+    program; what it queues depends on device memory only."""
+    b.call(getattr(kernels.lib(), "picolm_call_" + name), out=out, user=args, recordable=True, **kw)

@@ -14,8 +14,11 @@ from .base import Part, Runtime
 class TokenEmbedding(Part):
     graph_safe = True      # launches depend on device memory only
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0, keeps_output: bool = False):
+        """`scale`: the rows are multiplied by it (in float).  `keeps_output`: the output is also
+        left in a buffer of its own (`embed.out`), for parts that read it again later."""
         self.name, self.V, self.D = name, vocab_size, hidden_size
+        self.scale, self.keeps_output = float(scale), bool(keeps_output)
         self.table = None
 
     def tensor_specs(self):
@@ -30,19 +33,26 @@ class TokenEmbedding(Part):
         if self.table is None:
             raise ValueError(f"embedding {self.name} has no table loaded")
         x = b.buffer("residual", self.D, torch.float32)
-        b.embed(self.table, x)
+        b.embed(self.table, x, self.scale)
+        if self.keeps_output:
+            b.embed(self.table, b.buffer("embed.out", self.D, torch.float32), self.scale)
         return x
 
     def forward(self, tokens: torch.Tensor, x: torch.Tensor) -> None:
         """The same on tensors, now: rows of the table for `tokens`, widened to float, into x."""
         kernels.embed(self.table, tokens, x)
+        if self.scale != 1.0:
+            x.mul_(self.scale)
 
 
 class LMHead(Part):
     graph_safe = True      # launches depend on device memory only
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, embedding: TokenEmbedding, tied: bool):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, embedding: TokenEmbedding, tied: bool,
+                 softcap: float = 0.0):
+        """`softcap` c > 0: logits <- c tanh(logits / c)."""
         self.name, self.V, self.D, self.embedding, self.tied = name, vocab_size, hidden_size, embedding, tied
+        self.softcap = float(softcap or 0.0)
         self.weight = None
 
     def tensor_specs(self):
@@ -64,8 +74,14 @@ class LMHead(Part):
             raise ValueError(f"head {self.name} has no weights loaded")
         logits = b.buffer("logits", self.V, torch.float32, ROWS_WANTED)
         b.linear(self.weight, src, logits, kernels.EPI_STORE, rows=ROWS_WANTED)
+        if self.softcap > 0:
+            from .calls import MAP_SOFTCAP, MapRowsArgs, emit_library_call
+            from ..engine.program import F32
+            emit_library_call(b, "map_rows", MapRowsArgs(MAP_SOFTCAP, self.V, F32, F32, self.softcap), logits, rows=ROWS_WANTED)
         b.logits_buffer = logits
 
     def forward(self, h: torch.Tensor, logits: torch.Tensor) -> None:
         """The same on tensors, now."""
         kernels.gemm(h, self.weight, logits, kernels.EPI_STORE)
+        if self.softcap > 0:
+            logits.copy_(self.softcap * torch.tanh(logits / self.softcap))

@@ -35,3 +35,33 @@ class SwiGLU(FeedForward):
         act = ctx.ws.get("ffn.act", (h.shape[0], self.F), ctx.dtype)
         self.gate_up.forward(h, act, kernels.EPI_SWIGLU)
         self.down.forward(act, residual, kernels.EPI_ACCUMULATE)
+
+
+class ActivatedMLP(FeedForward):
+    """Two matrices with an activation between them: down(act(up h)), no bias.  `activation`:
+    "relu_squared" is max(z, 0)^2.  The up product leaves float rows, the activation is taken in
+    float and rounded once to the dtype the down product reads."""
+    graph_safe = True      # launches depend on device memory only
+    ACTIVATIONS = {"relu_squared": 1}
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "relu_squared",
+                 names=("up", "down")):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"activation '{activation}': known are {', '.join(self.ACTIVATIONS)}")
+        self.D, self.F, self.activation = hidden_size, intermediate_size, activation
+        self.up = Linear([prefix + names[0]], [intermediate_size], hidden_size)
+        self.down = Linear([prefix + names[1]], [hidden_size], intermediate_size)
+
+    def children(self):
+        return [self.up, self.down]
+
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0) -> None:
+        """x += down(act(up h)) for the rows h of `src`, as operations of a launch program."""
+        import torch
+        from ..engine.program import _DT, F32
+        from .calls import MapRowsArgs, emit_library_call
+        pre = b.buffer("ffn.pre", self.F, torch.float32)
+        act = b.buffer("ffn.act", self.F, b.dtype)
+        self.up.emit(b, src, pre, kernels.EPI_STORE)
+        emit_library_call(b, "map_rows", MapRowsArgs(self.ACTIVATIONS[self.activation], self.F, F32, _DT[b.dtype], 0.0), act, inp=pre)
+        self.down.emit(b, act, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)

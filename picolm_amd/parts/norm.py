@@ -22,7 +22,7 @@ class RMSNorm(Norm):
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name, (self.size,), init="ones")]
+        return [TensorSpec(self.name, (self.size,), init="zeros" if self.weight_offset == 1.0 else "ones")]
 
     def load(self, fetch, runtime: Runtime) -> None:
         w = fetch.get(self.name).to(torch.float32)      # exact; picolm converts norm weights at load too (model_core.c:947-995)

@@ -50,12 +50,13 @@ class WeightsError(ValueError):
 
 @dataclass(frozen=True)
 class TensorSpec:
-    """What a part needs from the checkpoint: a name, a shape, and whether it may be absent."""
+    """What a part needs from the checkpoint: a name, a shape (-1: this dimension is the tensor's
+    to say), and whether it may be absent."""
     name: str
     shape: tuple
     optional: bool = False
     kind: str = "float"          # "float" or "int"
-    init: str | None = "normal"  # random-weights mode: "normal", "ones", or None (not written)
+    init: str | None = "normal"  # random-weights mode: "normal", "ones", "zeros" (both with the norms' spread), or None (not written)
 
 
 def canonical_name(name: str) -> str:
@@ -165,7 +166,7 @@ def check_specs(source, specs: list[TensorSpec]) -> None:
         if n not in have:
             continue
         dtype, shape = source.info(n)
-        if tuple(shape) != tuple(s.shape):
+        if len(shape) != len(s.shape) or any(want != -1 and want != got for want, got in zip(s.shape, shape)):
             wrong_shape.append((n, tuple(s.shape), tuple(shape)))
         if stored_dtype(dtype, s.kind) is None:
             wrong_dtype.append((n, str(dtype).replace("torch.", "")))

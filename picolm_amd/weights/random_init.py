@@ -3,7 +3,7 @@
 picolm has nothing like it (nearest: `srand48(42)` blocks in its kernel diff,
 picolm/picolm.c:577-593).  Each tensor has a stream of its own, derived from the seed and
 the tensor's name, so a tensor's values do not depend on which others are made.  Matrices
-are N(0, std); norm weights are 1, or 1 + N(0, norm_sigma).
+are N(0, std); norm weights are 1 (0 where the norm adds one itself), or that plus N(0, norm_sigma).
 """
 from __future__ import annotations
 
@@ -29,8 +29,10 @@ def random_tensor(spec: TensorSpec, seed: int, std: float, norm_sigma: float,
     gen.manual_seed(_stream_seed(seed, spec.name))
     if spec.kind == "int":
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    if spec.init == "ones":
-        t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+    if any(int(n) < 0 for n in spec.shape):
+        raise ValueError(f"random weights: the shape of '{spec.name}' is left to the checkpoint; the configuration must name it")
+    if spec.init in ("ones", "zeros"):
+        t = torch.full(tuple(spec.shape), 1.0 if spec.init == "ones" else 0.0, dtype=torch.float32, device=device)
         if norm_sigma > 0:
             t += torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) * norm_sigma
     else:
