@@ -32,7 +32,7 @@ def parse_ids(text: str) -> list[int]:
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="picolm", description="Llama text generation on MI355X: token ids in, token ids out")
+    ap = argparse.ArgumentParser(prog="picolm", description="Text generation on MI355X: token ids in, token ids out")
     ap.add_argument("model", nargs="?", help="folder with config.json and model.safetensors")
     ap.add_argument("-p", dest="prompt", help="prompt as token ids (else standard input)")
     ap.add_argument("-n", dest="max_tokens", type=int, default=256, help="max tokens to generate (default 256)")
@@ -120,11 +120,13 @@ def main(argv=None) -> int:
         if bos is None:
             raise SystemExit("no prompt given, and this model's configuration names no start token (bos_token_id)")
         prompts = [[int(bos)]]
-    context = args.context or cfg.max_position_embeddings
+    # (a configuration without position tables names no longest sequence: the prompts and -n say)
+    longest = getattr(cfg, "max_position_embeddings", None) or max(len(p) for p in prompts) + args.max_tokens
+    context = args.context or longest
     params = SamplingParams(args.temperature, args.top_k, args.top_p, args.min_p, args.seed)
     if args.benchmark or args.benchmark_ctx:        # one sequence, speed only (picolm.c:969-976, :1311)
         from . import diagnostics
-        context = min(context, cfg.max_position_embeddings)
+        context = min(context, longest)
         session = Session(model, max_tokens=pages_for(context) * PAGE_TOKENS, max_seq_len=context, n_slots=1)
         if args.benchmark_ctx:
             return diagnostics.benchmark_ctx(session, prompts[0], args.max_tokens, context, params)
