@@ -154,6 +154,138 @@ def library_products(cfg, dev, prefill_rows: int) -> dict:
     return {"library_products": out, "model": "layer sizes of " + str(cfg.hidden_size) + " x " + str(cfg.intermediate_size)}
 
 
+# ---- another design beside the closest Llama of equal size --------------------------------------------
+def _begopel_pair(width: int, heads: int, kv_heads: int, ff: int, vocab: int, pairs: int, loop_times: int = 0):
+    """A Begopel of `pairs` (parallel, mamba2) pairs of layers with heads of 128, and the Llama of the
+    same width, heads, feed-forward width, vocabulary and number of layer runs."""
+    att = dict(heads=heads, kv_heads=kv_heads, dim=128, vdim=128, scale=128 ** -0.5, bias_max=4096.0, bias_rows=64)
+    delta = dict(heads=heads, kv_heads=max(heads // 2, 1), dim=128, vdim=128, conv=4)
+    mamba = dict(heads=2 * width // 64, vdim=64, state=128, groups=max(heads // 4, 1), norm_groups=1, conv=4)
+    mlp = dict(kind="dense", ff=ff)
+    layers = []
+    for _ in range(pairs):
+        layers += [dict(type="parallel", mixer=dict(left=att, right=delta), mlp=mlp), dict(type="mamba2", mixer=mamba, mlp=mlp)]
+    beg = dict(architecture="Begopel", vocab=vocab, width=width, embedding=dict(scale=1.0), norm=dict(eps=1e-6), layers=layers,
+               logit_softcap=30.0)
+    runs = 2 * pairs
+    if loop_times:
+        beg["loop"] = dict(start=0, stop=2, times=loop_times)
+        runs += 2 * (loop_times - 1)
+    llama = dict(architectures=["LlamaForCausalLM"], hidden_size=width, intermediate_size=ff, num_attention_heads=heads,
+                 num_key_value_heads=kv_heads, num_hidden_layers=runs, vocab_size=vocab, head_dim=128, rms_norm_eps=1e-6,
+                 rope_theta=500000.0, rope_scaling=None, tie_word_embeddings=True, max_position_embeddings=131072, eos_token_id=2)
+    return beg, llama
+
+
+DESIGN_SIZES = {
+    "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
+                ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
+}
+
+
+def _begopel_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
+    """Per label of operation, the seconds that the work of one prefill step of T tokens and of one
+    decode step of n_seq sequences at `context` would take at the peak that binds it: products and
+    softmax attention in a prefill at the bf16 matrix peak, the walk of a matrix state at the 32-bit
+    vector peak (its state is 32-bit and its recurrence is no product), everything in a decode step
+    and every row-wise operation at HBM's peak over the bytes it must move."""
+    runs = []
+    loop = cfg.get("loop")
+    for i, layer in enumerate(cfg["layers"]):
+        runs += [layer] * (loop["times"] if loop and loop["start"] <= i < loop["stop"] else 1)
+    mfma, valu, hbm = PEAK_TFLOPS["bf16"] * 1e12, PEAK_TFLOPS["fp32"] * 1e12, HBM_PEAK_GBS * 1e9
+    pre = {"sink_attention": 0.0, "state_scan": 0.0}
+    dec = {"sink_attention": 0.0, "state_scan": 0.0}
+    for layer in runs:
+        m = layer["mixer"]
+        if layer["type"] == "parallel":
+            l, r = m["left"], m["right"]
+            pre["sink_attention"] += 2.0 * l["heads"] * (l["dim"] + l["vdim"]) * (T * (T + 1) / 2) / mfma
+            dec["sink_attention"] += n_seq * context * l["kv_heads"] * (l["dim"] + l["vdim"]) * 2 / hbm
+            pre["state_scan"] += 7.0 * T * r["heads"] * r["dim"] * r["vdim"] / valu
+            dec["state_scan"] += n_seq * 2 * r["heads"] * r["dim"] * r["vdim"] * 4 / hbm
+        else:
+            pre["state_scan"] += 5.0 * T * m["heads"] * m["state"] * m["vdim"] / valu
+            dec["state_scan"] += n_seq * 2 * m["heads"] * m["state"] * m["vdim"] * 4 / hbm
+    return {"prefill": pre, "decode": dec}
+
+
+def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int) -> dict:
+    """Prefill and decode throughput of `design` at a few sizes that resemble real layers (random
+    weights), beside the Llama of equal size, and the GPU time of one prefill step and one decode
+    step by operation."""
+    import torch
+
+    from picolm_amd.config import BegopelConfig, LlamaConfig
+    from picolm_amd.engine import Session, random_model
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+    out = {"design": design, "prefill_tokens": T, "decode_batch": n_seq, "decode_context": context, "dtype": "bf16",
+           "data": "synthetic", "sizes": []}
+
+    def measure(cfg, vocab):
+        model = random_model(cfg, seed=0, std=0.02, dtype="bfloat16", device=dev)
+        prompt = [int(t) for t in rng.integers(0, vocab, size=T)]
+        res = {}
+        for timed in (False, True):
+            sess = Session(model, max_tokens=(T + 64) + n_seq * (context + 2 * steps + 64), n_slots=n_seq + 1, time_ops=timed)
+            times = []
+            for _ in range(4):
+                [s] = sess.begin(1)
+                torch.cuda.synchronize()
+                if timed:
+                    sess.engine.op_times()
+                t0 = time.perf_counter()
+                sess.step([s], [prompt])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                if timed:
+                    res["prefill_ops_ms"] = sess.engine.op_times_by_label()
+                sess.release([s])
+            if not timed:
+                res["prefill_tok_s"] = T / float(np.median(times[1:]))
+            slots = sess.begin(n_seq)
+            sess.step(slots, [[int(t) for t in rng.integers(0, vocab, size=context)] for _ in range(n_seq)])
+            toks = [[int(t)] for t in rng.integers(0, vocab, size=n_seq)]
+            for _ in range(4):
+                sess.step(slots, toks)
+            torch.cuda.synchronize()
+            if timed:
+                sess.engine.op_times()
+                sess.step(slots, toks)
+                res["decode_ops_ms"] = sess.engine.op_times_by_label()
+            else:
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    sess.step(slots, toks)
+                torch.cuda.synchronize()
+                res["decode_tok_s"] = n_seq * steps / (time.perf_counter() - t0)
+            sess.release(slots)
+            del sess
+            torch.cuda.empty_cache()
+        del model
+        torch.cuda.empty_cache()
+        return res
+
+    for name, size in DESIGN_SIZES[design]:
+        beg, llama = _begopel_pair(*size)
+        print(f"[bench] {design} {name}", file=sys.stderr, flush=True)
+        a = measure(BegopelConfig.from_dict(beg), beg["vocab"])
+        b = measure(LlamaConfig.from_dict(llama), llama["vocab_size"])
+        roof = _begopel_rooflines(beg, T, n_seq, context)
+        lc = LlamaConfig.from_dict(llama)
+        like = {"prefill": attention_flops(lc, T) / (PEAK_TFLOPS["bf16"] * 1e12),
+                "decode": n_seq * context * kv_bytes_per_token(lc) / (HBM_PEAK_GBS * 1e9)}
+        fractions = {}
+        for phase in ("prefill", "decode"):
+            ops = a[phase + "_ops_ms"]
+            fractions[phase] = {k: roof[phase][k] / (ops[k] * 1e-3) for k in roof[phase] if ops.get(k)}
+            fractions[phase]["llama attention"] = like[phase] / (b[phase + "_ops_ms"]["attention"] * 1e-3)
+        out["sizes"].append({"size": name, "layer_runs": llama["num_hidden_layers"], design: a, "llama": b,
+                             "fraction_of_roofline": fractions})
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -185,7 +317,13 @@ def main() -> int:
     ap.add_argument("--steps-ahead", type=int, choices=[0, 1], default=1,
                     help="1 (the generation loop's way): the next step is launched before this step's tokens are "
                          "read on the host; 0: the host reads every step's tokens first")
+    ap.add_argument("--design", choices=sorted(DESIGN_SIZES), default="",
+                    help="instead of the record: prefill and decode throughput of another design at a few sizes beside the "
+                         "Llama of equal size, with the GPU time of a step by operation, as one JSON line")
     args = ap.parse_args()
+    if args.design:
+        print(json.dumps(design_comparison(args.design, args.prefill_tokens, args.batch or 8, 1024, args.steps or 32)))
+        return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2

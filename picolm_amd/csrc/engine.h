@@ -238,6 +238,9 @@ int picolm_engine_generate(picolm_engine* e, int32_t n_prompts, const int32_t* p
 // and the cache write).  Waits for the GPU.  picolm prints such figures for its layers itself
 // (picolm/picolm.c:305-317).
 int picolm_engine_op_times(picolm_engine* e, double* ms);
+// The same by operation: each[i] is the time of the program's operation i (n_each = its number of
+// operations); either array may be null.
+int picolm_engine_op_times_each(picolm_engine* e, double* ms, double* each, int32_t n_each);
 
 // ---- what the engine holds, for bindings and tests ---------------------------------------------
 // what: 0 max_seq_len, 1 n_slots, 2 free slots, 3 free tokens (pages free in the tightest group

@@ -387,7 +387,7 @@ struct picolm_engine {
     const StepPlan* last_plan = nullptr;
     // timing by class of operation (PICOLM_ENGINE_TIME_OPS): an event before and after each one
     struct TimedOp {
-        int cls;
+        int cls, op;
         hipEvent_t before, after;
     };
     std::vector<TimedOp> timed;
@@ -1319,20 +1319,26 @@ static int run_program(picolm_engine* e, const StepPlan& p, Workspace& w, hipStr
             hipEvent_t after = nullptr;
             TRY(timing_event(e, &after, stream));
             const int cls = o.kind == PICOLM_OP_LINEAR ? (o.rows == PICOLM_ROWS_WANTED ? 2 : 1) : o.kind == PICOLM_OP_ATTENTION ? 3 : 0;
-            e->timed.push_back({cls, before, after});
+            e->timed.push_back({cls, (int)(&o - e->ops.data()), before, after});
         }
     }
     return 0;
 }
 
-extern "C" int picolm_engine_op_times(picolm_engine* e, double* ms) {
-    E_REQUIRE(-1, e && ms && e->timing(), "op_times: the engine was not made with PICOLM_ENGINE_TIME_OPS");
-    for (int c = 0; c < 4; ++c) ms[c] = 0.0;
+extern "C" int picolm_engine_op_times(picolm_engine* e, double* ms) { return picolm_engine_op_times_each(e, ms, nullptr, 0); }
+
+extern "C" int picolm_engine_op_times_each(picolm_engine* e, double* ms, double* each, int32_t n_each) {
+    E_REQUIRE(-1, e && (ms || each) && e->timing(), "op_times: the engine was not made with PICOLM_ENGINE_TIME_OPS");
+    E_REQUIRE(-1, !each || n_each == (int32_t)e->ops.size(), "op_times: the program has %d operations, the caller has room for %d",
+              (int)e->ops.size(), n_each);
+    for (int c = 0; ms && c < 4; ++c) ms[c] = 0.0;
+    for (int i = 0; each && i < n_each; ++i) each[i] = 0.0;
     for (auto& t : e->timed) {
         HIP_TRY(hipEventSynchronize(t.after));
         float dt = 0.f;
         HIP_TRY(hipEventElapsedTime(&dt, t.before, t.after));
-        ms[t.cls] += dt;
+        if (ms) ms[t.cls] += dt;
+        if (each) each[t.op] += dt;
         e->spare_events.push_back(t.before);
         e->spare_events.push_back(t.after);
     }

@@ -215,6 +215,20 @@ class NativeEngine:
             _raise(rc)
         return {"other": ms[0], "products": ms[1], "head": ms[2], "attention": ms[3]}
 
+    def op_times_by_label(self) -> dict:
+        """GPU milliseconds since the last call of this or of `op_times`, summed over the program's
+        operations of one label: a product's sizes, an engine operation's kind, or the name of a
+        called operation."""
+        n = self.program.n_ops
+        each = (ctypes.c_double * n)()
+        rc = _lib().picolm_engine_op_times_each(self.handle, None, each, n)
+        if rc:
+            _raise(rc)
+        out: dict = {}
+        for label, ms in zip(self.program.op_labels, each):
+            out[label] = out.get(label, 0.0) + ms
+        return out
+
     def step_array(self, name: str) -> np.ndarray:
         n = _lib().picolm_engine_step_array(self.handle, name.encode(), None, 0)
         if n < 0:

@@ -131,6 +131,7 @@ class ProgramBuilder:
         self.binding = None                   # the cache binding of the layer call being emitted
         self.logits_buffer = -1
         self.failures: list = []              # exceptions that called Python operations raised, newest last
+        self.labels: dict[int, str] = {}      # operation index -> what a part called it (for timings by operation)
 
     def buffer(self, name: str, width: int, dtype: torch.dtype, rows: int = ROWS_STEP) -> int:
         row_bytes = int(width) * dtype.itemsize
@@ -201,7 +202,7 @@ class ProgramBuilder:
 
     def call(self, fn, out: int, inp: int = -1, extra=(), rows: int = ROWS_STEP, user=None, recordable: bool = False,
              uses_kv: bool = False, attends: bool = False, uses_state: bool = False, tile_rows: int = 0,
-             partial_floats: int = 0) -> None:
+             partial_floats: int = 0, label: str | None = None) -> None:
         """An operation of the caller's.  `fn`: a C function `int (*)(void* user, const
         picolm_step_view*)` as a ctypes function pointer or address (with `user`, an address or a
         ctypes object that is kept alive), or a Python callable taking the `StepView`; it queues
@@ -237,6 +238,8 @@ class ProgramBuilder:
             op.kv_group, op.kv_entry, op.kv_writes = b.kv[0], b.kv[1], int(b.writes)
         if uses_state:
             op.state_group, op.state_entry = b.state
+        if label:
+            self.labels[len(self.ops)] = label
         self.ops.append(op)
 
     def _trampoline(self, fn):
@@ -283,6 +286,9 @@ class BuiltProgram:
                               n_kv_groups=len(kv), state_groups=self.state_groups, n_state_groups=len(st))
         self.buffer_names = dict(b._buffers)
         self.n_ops = len(b.ops)
+        kinds = {OP_EMBED: "embed", OP_RMSNORM: "rmsnorm", OP_LINEAR: "linear", OP_ATTENTION: "attention", OP_CALL: "call"}
+        self.op_labels = [b.labels.get(i) or (f"linear {op.n}x{op.k}" if op.kind == OP_LINEAR else kinds.get(op.kind, "?"))
+                          for i, op in enumerate(b.ops)]
         self.recordable = all(op.kind != OP_CALL or op.call_flags & CALL_RECORDABLE for op in b.ops)
 
 
@@ -305,6 +311,8 @@ def declare(lib) -> None:
     lib.picolm_engine_set_prefill_step_tokens.restype = ctypes.c_int
     lib.picolm_engine_op_times.argtypes = [E, c_void_p]
     lib.picolm_engine_op_times.restype = ctypes.c_int
+    lib.picolm_engine_op_times_each.argtypes = [E, c_void_p, c_void_p, c_int32]
+    lib.picolm_engine_op_times_each.restype = ctypes.c_int
     lib.picolm_engine_info.argtypes = [E, c_int32]
     lib.picolm_engine_info.restype = c_int64
     lib.picolm_engine_kv_entry.argtypes = [E, c_int32, c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64)]

@@ -55,4 +55,4 @@ SHORT_CONV_MAX_TAPS = 16
 def emit_library_call(b, name: str, args: Structure, out: int, **kw) -> None:
     """Appends the library's operation `name` (`picolm_call_<name>`) with its arguments to the
     program; what it queues depends on device memory only."""
-    b.call(getattr(kernels.lib(), "picolm_call_" + name), out=out, user=args, recordable=True, **kw)
+    b.call(getattr(kernels.lib(), "picolm_call_" + name), out=out, user=args, recordable=True, label=name, **kw)
