@@ -110,7 +110,7 @@ int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, void* C, int
 int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 // What the vector-ALU attention kernels take beside keys, values and a scale (all optional: zero
 // or null is "none"): values of a size of their own, a bias by distance added to the scaled score
-// (bias[min(n, bias_rows - 1)][head] for a key n positions back), a sink (exp(sink[head]) joins the
+// (bias[head][min(n, bias_rows - 1)] for a key n positions back), a sink (exp(sink[head]) joins the
 // softmax's denominator once, with no key and no value), and a gate (the output of head h is
 // multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows).
 typedef struct {
@@ -133,6 +133,18 @@ int picolm_attn_decode_plain(const void* q, const void* k_pages, const void* v_p
                              const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
                              const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
                              const picolm_attn_extras* x, hipStream_t stream);
+// The same on the matrix cores: bfloat16, keys and values of the sizes that picolm_attn_plain_mfma_takes
+// says, prefill tiles of picolm_attn_plain_mfma_tile_rows() rows, no window.
+int picolm_attn_plain_mfma_takes(int d, int dv);
+int picolm_attn_plain_mfma_tile_rows(void);
+int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, const int32_t* tile_seq,
+                                   const int32_t* tile_q0, int n_tiles, const int32_t* seq_slot, const int32_t* seq_pos0,
+                                   const int32_t* seq_nnew, const int32_t* cu_seqlens, const int32_t* page_table, int max_pages,
+                                   int ring_pages, int H, int G, int d, float scale, const picolm_attn_extras* x, hipStream_t stream);
+int picolm_attn_decode_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int n_seq,
+                                  const int32_t* chunk_list, int n_chunks, int pages_per_chunk, int max_splits, const int32_t* seq_pos0,
+                                  const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, float scale,
+                                  const picolm_attn_extras* x, hipStream_t stream);
 int picolm_attn_prefill_tile_rows(void);
 int picolm_attn_prefill_generic(const void* q, const void* k_pages, const void* v_pages, void* out,
                                 int dt, const int32_t* tile_seq, const int32_t* tile_q0, int n_tiles,

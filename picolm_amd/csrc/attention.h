@@ -41,9 +41,9 @@ struct AttnArgs {
     // launches.  With it the workgroup that finishes a sequence's last chunk combines the chunks
     // itself and no merge kernel runs; null: the merge kernel does.
     int32_t* chunks_done;
-    // vector-ALU kernel only, all optional (zero: absent):
+    // kernels over plain pages only (attention_generic.hip, attention_plain_mfma.hip), all optional (zero: absent):
     int dv;                     // size of a value where it is not that of a key: out and partial rows are [H][dv]
-    const float* bias;          // [bias_rows][H]: added to the scaled score of a key n positions back, row min(n, bias_rows - 1)
+    const float* bias;          // [H][bias_rows]: added to the scaled score of a key n positions back, entry min(n, bias_rows - 1)
     int bias_rows;
     const float* sink;          // [H]: exp(sink) joins the softmax's denominator once, with no key and no value
     const float* gate;          // float rows: the output of head h is multiplied by sigmoid(gate[token * gate_stride + h * dv + c])

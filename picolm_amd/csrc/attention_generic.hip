@@ -142,7 +142,7 @@ __global__ __launch_bounds__(AT_THREADS) void attn_tile_kernel(AttnArgs a) {
                 float sc = NEG_BIG;
                 if (vis) {
                     sc = s[i] * a.scale;
-                    if (a.bias) sc += a.bias[(size_t)min(qp - kpos, a.bias_rows - 1) * a.H + row_head[r]];
+                    if (a.bias) sc += a.bias[(size_t)row_head[r] * a.bias_rows + min(qp - kpos, a.bias_rows - 1)];
                 }
                 const float m_new = fmaxf(m_run[i], wave_max(sc));
                 const float p = vis ? expf(sc - m_new) : 0.f;
@@ -314,7 +314,7 @@ int check_decode_chunks(const char* who, const float* partial, const int32_t* ch
     return 0;
 }
 
-static int check_attn_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
+int check_attn_sizes(const char* who, int H, int G, int d, int max_pages, int ring_pages) {
     PICOLM_REQUIRE(H > 0 && G > 0 && H % G == 0, "%s: %d heads do not split over %d groups", who, H, G);
     PICOLM_REQUIRE(d >= 1 && d <= AT_MAX_D, "%s: head size %d is not in [1, %d]", who, d, AT_MAX_D);
     PICOLM_REQUIRE(max_pages > 0 && ring_pages > 0 && ring_pages <= max_pages,

@@ -29,15 +29,17 @@ int picolm_call_loop_input(void* user, const picolm_step_view* v);
 // sink and an output gate, each optional.
 //   in: float rows [in_stride] holding q [H d], k [G d], v [G dv] and the gate's pre-activations
 //   [H dv] at the offsets named; out: rows [H dv] in the engine's dtype; extra[0]: scratch rows
-//   [H d] in the engine's dtype.  Flags: PICOLM_CALL_KV | PICOLM_CALL_ATTENDS, tile_rows =
-//   picolm_attn_prefill_tile_rows(), partial_floats = H (dv + 2).  Pages are kept as plain arrays.
+//   [H d] in the engine's dtype.  Flags: PICOLM_CALL_KV | PICOLM_CALL_ATTENDS, partial_floats =
+//   H (dv + 2), tile_rows = picolm_attn_plain_mfma_tile_rows() where the engine runs in bfloat16 and
+//   picolm_attn_plain_mfma_takes(d, dv) (the matrix-core kernel then runs), else
+//   picolm_attn_prefill_tile_rows().  Pages are kept as plain arrays.
 typedef struct {
     int32_t n_heads, n_kv_heads, head_dim, v_head_dim;
     int32_t in_stride, q_off, k_off, v_off, gate_off;     // gate_off < 0: no gate
     float scale, eps;
     const float* q_norm;     // [head_dim] RMS norm of each query head (null: none), and of each key head
     const float* k_norm;
-    const float* bias;       // [bias_rows][H] by distance, the last row for every distance beyond; null: none
+    const float* bias;       // [H][bias_rows] by distance, the last entry for every distance beyond; null: none
     int32_t bias_rows;
     const float* sink;       // [H] or null
 } picolm_sink_attention_args;

@@ -124,6 +124,18 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     x.sink = a->sink;
     x.gate = a->gate_off >= 0 ? in + a->gate_off : nullptr;
     x.gate_stride = a->in_stride;
+    const bool mfma = dt == PICOLM_BF16 && picolm_attn_plain_mfma_takes(d, dv);
+    if (mfma && v->is_decode)
+        return picolm_attn_decode_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, v->n_seq, v->chunk_list, v->n_chunks,
+                                             v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H,
+                                             G, d, a->scale, &x, v->stream);
+    if (mfma) {
+        PICOLM_REQUIRE(v->tile_seq && v->tile_rows == picolm_attn_plain_mfma_tile_rows(), "sink_attention: the step has no tiles of %d rows",
+                       picolm_attn_plain_mfma_tile_rows());
+        return picolm_attn_prefill_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->tile_seq, v->tile_q0, v->n_tiles, v->seq_slot,
+                                              v->seq_pos0, v->seq_nnew, v->cu_seqlens, v->page_table, v->max_pages, v->ring_pages, H, G, d,
+                                              a->scale, &x, v->stream);
+    }
     if (v->is_decode)
         return picolm_attn_decode_plain(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, dt, v->n_seq, v->chunk_list, v->n_chunks,
                                         v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H, G, d,
@@ -429,6 +441,34 @@ __global__ void gated_norm_kernel(const float* __restrict__ x, const float* __re
     }
 }
 
+// the same with a workgroup per (row, part), for parts of a thousand columns and more
+template <typename T>
+__global__ __launch_bounds__(256) void gated_norm_wide_kernel(const float* __restrict__ x, const float* __restrict__ gate, int gate_stride,
+                                                              int gate_off, T* __restrict__ out, const float* __restrict__ weight,
+                                                              int weight_len, int width, int group, float eps, int gate_first) {
+    __shared__ float scratch[16];
+    const int n_groups = width / group;
+    const size_t row = blockIdx.x / n_groups;
+    const int c0 = (int)(blockIdx.x % n_groups) * group;
+    const float* xr = x + row * width + c0;
+    const float* gr = gate ? gate + row * gate_stride + gate_off + c0 : nullptr;
+    float ssq = 0.f;
+    for (int c = threadIdx.x; c < group; c += blockDim.x) {
+        float xv = xr[c];
+        if (gr && gate_first) xv *= silu_f(gr[c]);
+        ssq += xv * xv;
+    }
+    ssq = block_sum(ssq, scratch);
+    const float inv = 1.f / sqrtf(ssq / (float)group + eps);
+    for (int c = threadIdx.x; c < group; c += blockDim.x) {
+        float xv = xr[c];
+        if (gr && gate_first) xv *= silu_f(gr[c]);
+        float y = xv * inv * weight[(c0 + c) % weight_len];
+        if (gr && !gate_first) y *= silu_f(gr[c]);
+        out[row * width + c0 + c] = from_f32<T>(y);
+    }
+}
+
 extern "C" int picolm_call_gated_norm(void* user, const picolm_step_view* v) {
     const picolm_gated_norm_args* a = (const picolm_gated_norm_args*)user;
     VIEW_REQUIRE("gated_norm", v);
@@ -440,8 +480,20 @@ extern "C" int picolm_call_gated_norm(void* user, const picolm_step_view* v) {
                    "gated_norm: the gate's rows of %d floats do not hold %d at %d", a->gate_stride, a->width, a->gate_off);
     if (v->rows <= 0) return 0;
     const int64_t n_units = (int64_t)v->rows * (a->width / a->group);
+    PICOLM_REQUIRE(n_units < (1ll << 31), "gated_norm: %lld workgroups exceed the grid", (long long)n_units);
+    if (a->group >= 1024) {
+        if (v->dtype == PICOLM_F32)
+            gated_norm_wide_kernel<float><<<(unsigned)n_units, 256, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0], a->gate_stride,
+                                                                                    a->gate_off, (float*)v->out, a->weight, a->weight_len,
+                                                                                    a->width, a->group, a->eps, a->gate_first);
+        else
+            gated_norm_wide_kernel<bf16_t><<<(unsigned)n_units, 256, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0],
+                                                                                     a->gate_stride, a->gate_off, (bf16_t*)v->out, a->weight,
+                                                                                     a->weight_len, a->width, a->group, a->eps, a->gate_first);
+        PICOLM_LAUNCH_CHECK("gated_norm (wide)");
+        return 0;
+    }
     const int64_t blocks = ceil_div64(n_units, 4);
-    PICOLM_REQUIRE(blocks < (1ll << 31), "gated_norm: %lld workgroups exceed the grid", (long long)blocks);
     if (v->dtype == PICOLM_F32)
         gated_norm_kernel<float><<<(unsigned)blocks, 4 * WAVE, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0], a->gate_stride,
                                                                                a->gate_off, (float*)v->out, a->weight, a->weight_len, a->width,

@@ -9,7 +9,8 @@ values may have a size of their own, and the heads are gated before the output p
 
 The bias table has B rows: one per distance below B/2, then rows spaced evenly in the logarithm of
 the distance up to `bias_max`, the last row for everything beyond.  It is expanded once, at load,
-into one row per distance up to `bias_max`; the attention kernel indexes that by min(distance, last).
+into one entry per distance up to `bias_max` and per head; the attention kernels index that by
+min(distance, last).
 """
 from __future__ import annotations
 
@@ -84,7 +85,7 @@ class SinkAttention(Mixer):
         if self.has_bias:
             rel = f32("rel")
             rows = distance_rows(rel.shape[0], self.bias_max)
-            self.bias = rel[torch.tensor(rows, device=rel.device)].contiguous()       # [distances, H]
+            self.bias = rel[torch.tensor(rows, device=rel.device)].t().contiguous()   # [H, distances]
         if self.has_sink:
             self.sink = f32("sink")
 
@@ -102,9 +103,12 @@ class SinkAttention(Mixer):
         q_off, k_off, v_off = 0, H * d, H * d + G * d
         args = SinkAttentionArgs(H, G, d, dv, width, q_off, k_off, v_off, v_off + G * dv if self.has_gate else -1, self.scale, self.eps,
                                  b._ptr(self.q_norm), b._ptr(self.k_norm), b._ptr(self.bias),
-                                 0 if self.bias is None else self.bias.shape[0], b._ptr(self.sink))
+                                 0 if self.bias is None else self.bias.shape[1], b._ptr(self.sink))
+        lib = kernels.lib()
+        on_matrix_cores = b.dtype == torch.bfloat16 and lib.picolm_attn_plain_mfma_takes(d, dv)
         emit_library_call(b, "sink_attention", args, out, inp=rows, extra=[q], uses_kv=True, attends=True,
-                          tile_rows=kernels.attn_prefill_tile_rows(), partial_floats=H * (dv + 2))
+                          tile_rows=lib.picolm_attn_plain_mfma_tile_rows() if on_matrix_cores else kernels.attn_prefill_tile_rows(),
+                          partial_floats=H * (dv + 2))
         if accumulate:
             self.o.emit(b, out, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)
         else:

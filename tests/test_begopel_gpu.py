@@ -79,7 +79,11 @@ ALONE = {
     "attention": (one_layer(bt.parallel(bt.attention(4, 2, 12, 20, 0.6, 25.0, 10), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
     "delta": (one_layer(bt.parallel(bt.attention(2, 1, 8, 8, 0.3, 9.0, 4), bt.delta(6, 2, 20, 12, 3), None)), "left.out"),
     "both": (one_layer(bt.parallel(bt.attention(3, 1, 16, 24, 0.4, 12.0, 8), bt.delta(3, 3, 12, 28, 4), None)), None),
+    # head sizes that the matrix-core attention takes in bfloat16 (64, 96, 128 on either side), with more than 32 heads a group
+    "attention, sizes of real heads": (one_layer(bt.parallel(bt.attention(4, 2, 96, 64, 0.2, 25.0, 10), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
+    "attention, forty heads a group": (one_layer(bt.parallel(bt.attention(40, 1, 64, 128, 0.25, 70.0, 16), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
     "mamba": (one_layer(bt.mamba(6, 8, 12, 3, 2, 3, None)), None),
+    "mamba, a wide norm": (one_layer(bt.mamba(20, 64, 8, 1, 1, 2, None)), None),
     "mamba, one tap": (one_layer(bt.mamba(2, 24, 20, 1, 3, 1, None)), None),
     "feed-forward": (one_layer(bt.mamba(1, 16, 8, 1, 1, 2, 80)), None),
     "loop": (one_layer(bt.mamba(2, 8, 8, 2, 1, 2, 24), loop=(0, 1, 3)), None),
@@ -224,21 +228,21 @@ def test_slots_and_pages_that_are_used_again(dtype):
 
 
 # ------------------------------------------------------------------------------ far keys, edges of the table and of pages
-def lookup_model(bias_max, bias_rows, heads=2, kv_heads=1):
+def lookup_model(bias_max, bias_rows, heads=2, kv_heads=1, dim=32, vdim=16):
     """One attention layer that looks a token's partner up.  Queries and keys share their matrix and
     read the first half of the width only, values read the second half, and token t + 700 has the
     first half of token t's embedding: so the score of t against t + 700 is as high as against
     itself, wherever the partner stands, while the partner's value is its own.  The delta branch is
     silenced.  In a sequence of otherwise unrelated tokens, about half of the last token's attention
     rests on the one key of its partner, more or less by the bias of that distance."""
-    cfg = bt.config(1400, 64, [bt.parallel(bt.attention(heads, kv_heads, 32, 16, 1.0, bias_max, bias_rows), bt.delta(2, 2, 8, 8, 2), None)],
-                    scale=2.0)
+    cfg = bt.config(1400, 64, [bt.parallel(bt.attention(heads, kv_heads, dim, vdim, 32.0 / dim, bias_max, bias_rows), bt.delta(2, 2, 8, 8, 2),
+                                           None)], scale=2.0)
     w = bt.make_weights(cfg, 5)
     w["embed"][700:, :32] = w["embed"][:700, :32]
     w["l0.mix.left.k"][:, 32:] = 0
     w["l0.mix.left.v"][:, :32] = 0
     w["l0.mix.left.q"] = w["l0.mix.left.k"].repeat(heads // kv_heads, 1)
-    w["l0.mix.left.q.norm"] = w["l0.mix.left.k.norm"] = torch.ones(32, dtype=torch.bfloat16)
+    w["l0.mix.left.q.norm"] = w["l0.mix.left.k.norm"] = torch.ones(dim, dtype=torch.bfloat16)
     w["l0.mix.right.out"] = torch.zeros_like(w["l0.mix.right.out"])
     w["l0.mix.left.sink"] = torch.full_like(w["l0.mix.left.sink"], 31.0)       # of the size of a match's score (32): it counts
     w["l0.mix.left.rel"] = (0.7 * torch.randn(bias_rows, heads, generator=torch.Generator().manual_seed(1))).to(torch.bfloat16)
@@ -257,20 +261,22 @@ _FAR, _EDGES = {}, {}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_one_far_key_among_hundreds(dtype):
+@pytest.mark.parametrize("dims", [(32, 16), (64, 64)])
+def test_one_far_key_among_hundreds(dims, dtype):
     """The asking token is the last; the key it asks for lies hundreds back, at the first places of
-    the sequence, and just before and after page borders.  Both in a prompt and decoded."""
-    cfg, w = lookup_model(40.0, 8)
+    the sequence, and just before and after page borders.  Both in a prompt and decoded.  (Heads of
+    64 go through the matrix-core kernel in bfloat16.)"""
+    cfg, w = lookup_model(40.0, 8, dim=dims[0], vdim=dims[1])
     model = bt.load(cfg, w, dtype)
     s = new_session(model, 2048)
     n = 500
     for needle_at in (0, 1, 63, 64, 65, 128, 383, 498):
         tokens = distinct_tokens(n, needle_at, cfg["vocab"], needle_at)
-        if needle_at not in _FAR:
+        if (dims, needle_at) not in _FAR:
             other = list(tokens)
             other[needle_at] = next(t for t in range(cfg["vocab"] // 2) if t not in tokens)
-            _FAR[needle_at] = (bt.plain_logits(cfg, w, tokens)[-1], bt.plain_logits(cfg, w, other)[-1])
-        want, missed = _FAR[needle_at]
+            _FAR[(dims, needle_at)] = (bt.plain_logits(cfg, w, tokens)[-1], bt.plain_logits(cfg, w, other)[-1])
+        want, missed = _FAR[(dims, needle_at)]
         assert bt.distance(missed, want) > 0.1, "the key must count"
         [slot] = s.begin(1)
         got = s.step([slot], [tokens]).double().cpu().numpy()
@@ -284,12 +290,12 @@ def test_one_far_key_among_hundreds(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("bias_max,bias_rows", [(40.0, 8), (17.5, 6), (100.0, 32)])
-def test_every_distance_across_the_tables_edges(bias_max, bias_rows, dtype):
+@pytest.mark.parametrize("bias_max,bias_rows,dims", [(40.0, 8, (32, 16)), (17.5, 6, (32, 16)), (100.0, 32, (32, 16)), (40.0, 8, (128, 64))])
+def test_every_distance_across_the_tables_edges(bias_max, bias_rows, dims, dtype):
     """The asked key at every distance from 0 to beyond the table's reach: each row's first and last
     distance is among them.  The rows differ by about 0.5 in the score, which moves the logits by far
     more than the limit."""
-    cfg, w = lookup_model(bias_max, bias_rows)
+    cfg, w = lookup_model(bias_max, bias_rows, dim=dims[0], vdim=dims[1])
     model = bt.load(cfg, w, dtype)
     s = new_session(model, 1024)
     n = int(bias_max) + 12
@@ -298,7 +304,7 @@ def test_every_distance_across_the_tables_edges(bias_max, bias_rows, dtype):
     for back in range(1, n):
         tokens = distinct_tokens(n, n - 1 - back, cfg["vocab"], back)
         rows_seen.add(P.distance_bucket(back, bias_rows, bias_max))
-        key = (bias_max, bias_rows, back)
+        key = (bias_max, bias_rows, dims, back)
         if key not in _EDGES:
             _EDGES[key] = bt.plain_logits(cfg, w, tokens)[-1]
         want = _EDGES[key]
