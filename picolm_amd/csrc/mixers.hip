@@ -266,7 +266,20 @@ struct ScanArgs {
     int qkv_stride, q_off, k_off, v_off;
     int rule, heads, key_heads, key_dim, value_dim;
     int R, kpt, n_waves, n_cb;
+    // mode 0: whole sequences, from and to the slot's state.  A long prompt is walked in chunks of
+    // chunk_len tokens side by side instead: mode 1 leaves every chunk's effect on a state as
+    // (N, M) with  S_end = M S_start + N  (the update is affine in S: the chunk is walked once from
+    // S = 0 with its values, which gives N, and with the delta rule once more from S = I without
+    // values, which gives M as key_dim more columns; the outer-product rule's M is the product of
+    // the chunk's decays); scan_carry_kernel then takes the states from chunk to chunk; mode 3
+    // walks every chunk from its start state and writes the outputs.
+    int mode, chunk_len, chunks_per_seq, ws_cols;
+    float* ws;          // [sequence][chunk][head][key_dim][ws_cols]: N | M | S_start
 };
+
+__device__ __forceinline__ float* scan_ws(const ScanArgs& a, int seq, int chunk, int head) {
+    return a.ws + (((size_t)seq * a.chunks_per_seq + chunk) * a.heads + head) * a.key_dim * a.ws_cols;
+}
 
 // One workgroup per (sequence, head, block of value columns).  A column of the state lies in the
 // registers of R lanes (row i R + r with lane r), so that both sums over the rows of a column, the
@@ -280,19 +293,30 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
     float* vs = qs + SCAN_TB * kd;           // [TB][CB]
     float* aws = vs + SCAN_TB * CB;          // [TB][2]
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-    const int cb = blockIdx.x % a.n_cb, head = (blockIdx.x / a.n_cb) % a.heads, seq = blockIdx.x / (a.n_cb * a.heads);
+    const int cb = blockIdx.x % a.n_cb, head = (blockIdx.x / a.n_cb) % a.heads, unit = blockIdx.x / (a.n_cb * a.heads);
+    const int seq = a.mode ? unit / a.chunks_per_seq : unit, chunk = a.mode ? unit % a.chunks_per_seq : 0;
+    int row0 = a.cu_seqlens[seq], row1 = a.cu_seqlens[seq + 1];
+    if (a.mode) {
+        row0 += chunk * a.chunk_len;
+        if (row0 >= row1) return;               // (the whole workgroup: the sequence has fewer chunks)
+        row1 = min(row1, row0 + a.chunk_len);
+    }
     const int r = lane / CW, col = wave * CW + lane % CW, j = cb * CB + col;
-    const bool valid = j < a.value_dim;
+    const int n_cols = a.mode == 1 ? a.ws_cols - a.value_dim : a.value_dim;      // mode 1: the columns of N and of M
+    const bool valid = j < n_cols;
     const int kh = head / (a.heads / a.key_heads);
     float* st = a.state + (size_t)a.seq_slot[seq] * a.slot_floats + (size_t)head * a.key_dim * a.value_dim;
+    float* ws = a.mode ? scan_ws(a, seq, chunk, head) : nullptr;
     float S[SCAN_KPT];
 #pragma unroll
     for (int i = 0; i < SCAN_KPT; ++i) {
         const int kr = i * R + r;
-        S[i] = i < kpt && valid && kr < a.key_dim ? st[(size_t)kr * a.value_dim + j] : 0.f;
+        const bool in = i < kpt && valid && kr < a.key_dim;
+        if (a.mode == 0) S[i] = in ? st[(size_t)kr * a.value_dim + j] : 0.f;
+        else if (a.mode == 1) S[i] = in && j - a.value_dim == kr ? 1.f : 0.f;
+        else S[i] = in ? ws[(size_t)kr * a.ws_cols + (a.ws_cols - a.value_dim) + j] : 0.f;
     }
     const float skip = a.skip ? a.skip[head] : 0.f;
-    const int row0 = a.cu_seqlens[seq], row1 = a.cu_seqlens[seq + 1];
     for (int b0 = row0; b0 < row1; b0 += SCAN_TB) {
         const int nb = min(SCAN_TB, row1 - b0);
         __syncthreads();
@@ -340,15 +364,94 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
                     }
             }
             for (int off = CW; off < WAVE; off <<= 1) o += __shfl_xor(o, off, WAVE);
-            if (r == 0 && valid) a.out[(size_t)(b0 + t) * a.heads * a.value_dim + (size_t)head * a.value_dim + j] = o + skip * vv;
+            if (r == 0 && valid && a.mode != 1)
+                a.out[(size_t)(b0 + t) * a.heads * a.value_dim + (size_t)head * a.value_dim + j] = o + skip * vv;
         }
     }
+    if (a.mode == 3) return;
 #pragma unroll
     for (int i = 0; i < SCAN_KPT; ++i) {
         const int kr = i * R + r;
-        if (i < kpt && valid && kr < a.key_dim) st[(size_t)kr * a.value_dim + j] = S[i];
+        if (i < kpt && valid && kr < a.key_dim) {
+            if (a.mode == 0) st[(size_t)kr * a.value_dim + j] = S[i];
+            else ws[(size_t)kr * a.ws_cols + j] = S[i];
+        }
     }
 }
+
+// From chunk to chunk: S_start of every chunk, and the state after the last one to the slot.  One
+// workgroup per (sequence, head, CARRY_COLS value columns); the columns of S lie in LDS.
+#define CARRY_COLS 16
+#define CARRY_MAX (PICOLM_STATE_SCAN_MAX_KEY_DIM * CARRY_COLS / 256)      // elements a thread holds
+__global__ __launch_bounds__(256) void scan_carry_kernel(ScanArgs a) {
+    extern __shared__ float carry_lds[];      // [key_dim][CARRY_COLS]
+    const int n_cb = (a.value_dim + CARRY_COLS - 1) / CARRY_COLS;
+    const int cb = blockIdx.x % n_cb, head = (blockIdx.x / n_cb) % a.heads, seq = blockIdx.x / (n_cb * a.heads);
+    const int row0 = a.cu_seqlens[seq], row1 = a.cu_seqlens[seq + 1];
+    const int n_chunks = (row1 - row0 + a.chunk_len - 1) / a.chunk_len;
+    const int n_elem = a.key_dim * CARRY_COLS, s_off = a.ws_cols - a.value_dim;
+    float* st = a.state + (size_t)a.seq_slot[seq] * a.slot_floats + (size_t)head * a.key_dim * a.value_dim;
+    float next[CARRY_MAX];
+    for (int e = threadIdx.x; e < n_elem; e += 256) {
+        const int i = e / CARRY_COLS, j = cb * CARRY_COLS + e % CARRY_COLS;
+        carry_lds[e] = j < a.value_dim ? st[(size_t)i * a.value_dim + j] : 0.f;
+    }
+    __syncthreads();
+    for (int c = 0; c < n_chunks; ++c) {
+        float* ws = scan_ws(a, seq, c, head);
+        float decay = 1.f;
+        if (a.rule == 0) {
+            const int t0 = row0 + c * a.chunk_len, t1 = min(row1, t0 + a.chunk_len);
+            for (int t = t0; t < t1; ++t) decay *= a.aw[(size_t)t * 2 * a.heads + head];
+        }
+#pragma unroll
+        for (int n = 0; n < CARRY_MAX; ++n) {
+            const int e = threadIdx.x + n * 256;
+            if (e >= n_elem) break;
+            const int i = e / CARRY_COLS, jj = e % CARRY_COLS, j = cb * CARRY_COLS + jj;
+            const float s = carry_lds[e];
+            if (j < a.value_dim) ws[(size_t)i * a.ws_cols + s_off + j] = s;
+            float acc = j < a.value_dim ? ws[(size_t)i * a.ws_cols + j] : 0.f;
+            if (a.rule == 0) {
+                acc += decay * s;
+            } else {
+                const float* m = ws + (size_t)i * a.ws_cols + a.value_dim;
+                for (int k = 0; k < a.key_dim; ++k) acc += m[k] * carry_lds[k * CARRY_COLS + jj];
+            }
+            next[n] = acc;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < CARRY_MAX; ++n) {
+            const int e = threadIdx.x + n * 256;
+            if (e < n_elem) carry_lds[e] = next[n];
+        }
+        __syncthreads();
+    }
+    for (int e = threadIdx.x; e < n_elem; e += 256) {
+        const int i = e / CARRY_COLS, j = cb * CARRY_COLS + e % CARRY_COLS;
+        if (j < a.value_dim) st[(size_t)i * a.value_dim + j] = carry_lds[e];
+    }
+}
+
+// scratch of the chunked walk: one allocation of the process that grows to the largest request
+// (prefill steps are not recorded, so it never changes under a recorded step)
+static float* g_scan_ws = nullptr;
+static size_t g_scan_ws_floats = 0;
+static int scan_workspace(size_t floats, float** out) {
+    if (floats > g_scan_ws_floats) {
+        hipError_t e = g_scan_ws ? hipFree(g_scan_ws) : hipSuccess;
+        g_scan_ws = nullptr, g_scan_ws_floats = 0;
+        if (e == hipSuccess) e = hipMalloc((void**)&g_scan_ws, floats * sizeof(float));
+        PICOLM_REQUIRE(e == hipSuccess, "state_scan: %zu bytes of scratch for the chunked walk: %s", floats * sizeof(float), hipGetErrorString(e));
+        g_scan_ws_floats = floats;
+    }
+    *out = g_scan_ws;
+    return 0;
+}
+#define SCAN_CHUNK_TOKENS 64            // a chunk of the chunked walk, doubled while the scratch would pass the limit
+#define SCAN_CHUNKED_FROM 256           // new tokens of a sequence from which a step is walked in chunks
+#define SCAN_WS_LIMIT_FLOATS ((size_t)1 << 30)
 
 extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
     const picolm_state_scan_args* a = (const picolm_state_scan_args*)user;
@@ -396,18 +499,42 @@ extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
     while (R * SCAN_KPT < kd) R *= 2;
     s.R = R;
     s.kpt = ceil_div(kd, R);
+    s.mode = 0, s.chunk_len = 0, s.chunks_per_seq = 1, s.ws_cols = 0, s.ws = nullptr;
     const int CW = WAVE / R;
-    // few sequences: one wave a workgroup, so that more workgroups share the walk; many: up to four
-    int n_waves = std::min(4, ceil_div(vd, CW));
-    if ((int64_t)v->n_seq * heads * ceil_div(vd, n_waves * CW) < 1024) n_waves = 1;
-    s.n_waves = n_waves;
-    s.n_cb = ceil_div(vd, n_waves * CW);
-    const int64_t blocks = (int64_t)v->n_seq * heads * s.n_cb;
-    PICOLM_REQUIRE(blocks < (1ll << 31), "state_scan: %lld workgroups exceed the grid", (long long)blocks);
-    const size_t lds = sizeof(float) * SCAN_TB * ((size_t)2 * s.kpt * R + n_waves * CW + 2);
-    state_scan_kernel<<<(unsigned)blocks, n_waves * WAVE, lds, v->stream>>>(s);
-    PICOLM_LAUNCH_CHECK("state_scan");
-    return 0;
+    auto launch = [&](int units, int n_cols) -> int {
+        // few units: one wave a workgroup, so that more workgroups share the walk; many: up to four
+        int n_waves = std::min(4, ceil_div(n_cols, CW));
+        if ((int64_t)units * heads * ceil_div(n_cols, n_waves * CW) < 1024) n_waves = 1;
+        s.n_waves = n_waves;
+        s.n_cb = ceil_div(n_cols, n_waves * CW);
+        const int64_t blocks = (int64_t)units * heads * s.n_cb;
+        PICOLM_REQUIRE(blocks < (1ll << 31), "state_scan: %lld workgroups exceed the grid", (long long)blocks);
+        const size_t lds = sizeof(float) * SCAN_TB * ((size_t)2 * s.kpt * R + n_waves * CW + 2);
+        state_scan_kernel<<<(unsigned)blocks, n_waves * WAVE, lds, v->stream>>>(s);
+        PICOLM_LAUNCH_CHECK("state_scan");
+        return 0;
+    };
+    int most_new = 0;
+    if (!v->is_decode && !v->recording && v->n_new)
+        for (int i = 0; i < v->n_seq; ++i) most_new = std::max(most_new, v->n_new[i]);
+    if (most_new < SCAN_CHUNKED_FROM) return launch(v->n_seq, vd);
+    // the chunked walk of a long prompt
+    s.ws_cols = 2 * vd + (a->rule == 1 ? kd : 0);
+    s.chunk_len = SCAN_CHUNK_TOKENS;
+    auto ws_floats = [&]() { return (size_t)v->n_seq * ceil_div(most_new, s.chunk_len) * heads * kd * s.ws_cols; };
+    while (ws_floats() > SCAN_WS_LIMIT_FLOATS && s.chunk_len < most_new) s.chunk_len *= 2;
+    s.chunks_per_seq = ceil_div(most_new, s.chunk_len);
+    if (s.chunks_per_seq < 2) return launch(v->n_seq, vd);
+    if (scan_workspace(ws_floats(), &s.ws)) return -1;
+    PICOLM_REQUIRE((int64_t)v->n_seq * s.chunks_per_seq < (1 << 24), "state_scan: %d sequences of %d chunks", v->n_seq, s.chunks_per_seq);
+    s.mode = 1;
+    if (launch(v->n_seq * s.chunks_per_seq, s.ws_cols - vd)) return -1;
+    const int64_t carry_blocks = (int64_t)v->n_seq * heads * ceil_div(vd, CARRY_COLS);
+    PICOLM_REQUIRE(carry_blocks < (1ll << 31), "state_scan: %lld workgroups exceed the grid", (long long)carry_blocks);
+    scan_carry_kernel<<<(unsigned)carry_blocks, 256, sizeof(float) * kd * CARRY_COLS, v->stream>>>(s);
+    PICOLM_LAUNCH_CHECK("state_scan (carry)");
+    s.mode = 3;
+    return launch(v->n_seq * s.chunks_per_seq, vd);
 }
 
 // ---- RMS norm in equal parts of a row, with a gate ---------------------------------------------------

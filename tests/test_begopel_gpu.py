@@ -170,6 +170,39 @@ def test_portions_equal_the_whole_prompt_beyond_rounding(dtype):
     assert bt.distance(np.concatenate(parts), whole) <= (1e-5 if dtype == "float32" else 0.03)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["P", "Q", "R"])
+def test_long_prompts_walked_in_chunks(which, dtype):
+    """From 256 new tokens of a sequence on, the matrix states are walked in chunks of 64 side by
+    side (every chunk's effect on a state first, then the states from chunk to chunk, then the
+    outputs): a long prompt whole, in two long portions onto each other, and in a batch with a short
+    one and one that is a token over the threshold, then decoded on."""
+    cfg, w, model = model_of(which, dtype)
+    tokens = tokens_for(cfg, 645, 8)
+    want = truth_of(which, 0, tokens)
+    s = new_session(model, 2048)
+    assert bt.distance(run_whole(s, tokens[:641]), want[:641]) <= bt.LIMIT[dtype]
+    [slot] = s.begin(1)
+    rows = [0, 63, 64, 255, 256, 299]
+    got = s.step([slot], [tokens[:300]], [rows]).double().cpu().numpy()
+    assert bt.distance(got, want[rows]) <= bt.LIMIT[dtype]
+    got = s.step([slot], [tokens[300:641]], [list(range(341))]).double().cpu().numpy()
+    assert bt.distance(got, want[300:641]) <= bt.LIMIT[dtype]
+    for i in range(641, 645):
+        got = s.step([slot], [[tokens[i]]]).double().cpu().numpy()
+        assert bt.distance(got, want[i]) <= bt.LIMIT[dtype], ("decoded", i)
+    s.release([slot])
+    others = [tokens_for(cfg, n, 30 + n) for n in (10, 257)]
+    slots = s.begin(3)
+    got = s.step(slots, [tokens[:400]] + others).double().cpu().numpy()
+    assert bt.distance(got[0], want[399]) <= bt.LIMIT[dtype]
+    for i, q in enumerate(others):
+        assert bt.distance(got[1 + i], truth_of(which, 0, q)[-1]) <= bt.LIMIT[dtype], ("beside the long one", i)
+    got = s.step(slots[:1], [[tokens[400]]]).double().cpu().numpy()
+    assert bt.distance(got, want[400]) <= bt.LIMIT[dtype]
+    s.release(slots)
+
+
 # ------------------------------------------------------------------------------ batches
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("which", ["P", "Q"])
