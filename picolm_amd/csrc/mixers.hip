@@ -251,8 +251,7 @@ __global__ void state_scan_prepare_kernel(const float* __restrict__ in, int in_s
     }
 }
 
-#define SCAN_KPT 16      // rows of the state a thread keeps in registers
-#define SCAN_TB 8        // tokens whose q, k, v wait in LDS at a time
+#define SCAN_TB 16       // tokens whose q, k, v wait in LDS at a time
 
 struct ScanArgs {
     const float* qkv;
@@ -282,12 +281,17 @@ __device__ __forceinline__ float* scan_ws(const ScanArgs& a, int seq, int chunk,
 }
 
 // One workgroup per (sequence, head, block of value columns).  A column of the state lies in the
-// registers of R lanes (row i R + r with lane r), so that both sums over the rows of a column, the
-// read-back along k and the read-out along q, are a few steps across lanes.  Lane = r * CW + column
-// within the wave (CW = 64 / R columns a wave).
+// registers of R lanes, up to SCAN_KPT rows each (row i R + r with lane r), so that both sums over
+// the rows of a column, the read-back along k and the read-out along q, are short chains in a lane
+// and a few steps across lanes.  (A whole column of 128 rows in one lane was measured too: the
+// chains of 128 dependent multiply-adds and the fewer waves made the walk 2.4 times slower.)
+// Lane = r * CW + column within the wave (CW = 64 / R columns a wave).
+#define SCAN_KPT 16      // rows of the state a thread keeps in registers
+template <int R>
 __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
     extern __shared__ float scan_lds[];
-    const int R = a.R, CW = WAVE / R, kpt = a.kpt, kd = kpt * R, CB = a.n_waves * CW;
+    constexpr int CW = WAVE / R;
+    const int kpt = a.kpt, kd = kpt * R, CB = a.n_waves * CW;
     float* ks = scan_lds;                    // [TB][kd]
     float* qs = ks + SCAN_TB * kd;           // [TB][kd]
     float* vs = qs + SCAN_TB * kd;           // [TB][CB]
@@ -496,7 +500,7 @@ extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
     s.key_dim = kd;
     s.value_dim = vd;
     int R = 1;
-    while (R * SCAN_KPT < kd) R *= 2;
+    while (R * SCAN_KPT < kd) R *= 2;           // (up to 16 for keys of PICOLM_STATE_SCAN_MAX_KEY_DIM = 256)
     s.R = R;
     s.kpt = ceil_div(kd, R);
     s.mode = 0, s.chunk_len = 0, s.chunks_per_seq = 1, s.ws_cols = 0, s.ws = nullptr;
@@ -510,7 +514,12 @@ extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
         const int64_t blocks = (int64_t)units * heads * s.n_cb;
         PICOLM_REQUIRE(blocks < (1ll << 31), "state_scan: %lld workgroups exceed the grid", (long long)blocks);
         const size_t lds = sizeof(float) * SCAN_TB * ((size_t)2 * s.kpt * R + n_waves * CW + 2);
-        state_scan_kernel<<<(unsigned)blocks, n_waves * WAVE, lds, v->stream>>>(s);
+        const dim3 grid((unsigned)blocks), block(n_waves * WAVE);
+        if (R == 1) state_scan_kernel<1><<<grid, block, lds, v->stream>>>(s);
+        else if (R == 2) state_scan_kernel<2><<<grid, block, lds, v->stream>>>(s);
+        else if (R == 4) state_scan_kernel<4><<<grid, block, lds, v->stream>>>(s);
+        else if (R == 8) state_scan_kernel<8><<<grid, block, lds, v->stream>>>(s);
+        else state_scan_kernel<16><<<grid, block, lds, v->stream>>>(s);
         PICOLM_LAUNCH_CHECK("state_scan");
         return 0;
     };
