@@ -384,11 +384,16 @@ __global__ __launch_bounds__(256) void state_scan_kernel(ScanArgs a) {
 }
 
 // From chunk to chunk: S_start of every chunk, and the state after the last one to the slot.  One
-// workgroup per (sequence, head, CARRY_COLS value columns); the columns of S lie in LDS.
-#define CARRY_COLS 16
+// workgroup per (sequence, head, CARRY_COLS value columns); the columns of S lie in LDS.  Few
+// columns a workgroup, so that many workgroups share the one walk that is left in order.  The
+// outer-product rule's decays of all chunks are multiplied up first, a wave a chunk.  (The delta
+// rule's M passed through LDS in tiles of 32 columns was measured too: three times slower than rows
+// of M read from global memory by the threads that share them.)
+#define CARRY_COLS 4
 #define CARRY_MAX (PICOLM_STATE_SCAN_MAX_KEY_DIM * CARRY_COLS / 256)      // elements a thread holds
 __global__ __launch_bounds__(256) void scan_carry_kernel(ScanArgs a) {
-    extern __shared__ float carry_lds[];      // [key_dim][CARRY_COLS]
+    extern __shared__ float carry_lds[];      // S [key_dim][CARRY_COLS] | decays [chunks_per_seq]
+    float* decays = carry_lds + a.key_dim * CARRY_COLS;
     const int n_cb = (a.value_dim + CARRY_COLS - 1) / CARRY_COLS;
     const int cb = blockIdx.x % n_cb, head = (blockIdx.x / n_cb) % a.heads, seq = blockIdx.x / (n_cb * a.heads);
     const int row0 = a.cu_seqlens[seq], row1 = a.cu_seqlens[seq + 1];
@@ -400,29 +405,46 @@ __global__ __launch_bounds__(256) void scan_carry_kernel(ScanArgs a) {
         const int i = e / CARRY_COLS, j = cb * CARRY_COLS + e % CARRY_COLS;
         carry_lds[e] = j < a.value_dim ? st[(size_t)i * a.value_dim + j] : 0.f;
     }
+    if (a.rule == 0) {
+        const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+        for (int c = wave; c < n_chunks; c += 256 / WAVE) {
+            const int t0 = row0 + c * a.chunk_len, t1 = min(row1, t0 + a.chunk_len);
+            float p = 1.f;
+            for (int t = t0 + lane; t < t1; t += WAVE) p *= a.aw[(size_t)t * 2 * a.heads + head];
+            for (int off = 1; off < WAVE; off <<= 1) p *= __shfl_xor(p, off, WAVE);
+            if (lane == 0) decays[c] = p;
+        }
+    }
     __syncthreads();
     for (int c = 0; c < n_chunks; ++c) {
         float* ws = scan_ws(a, seq, c, head);
-        float decay = 1.f;
-        if (a.rule == 0) {
-            const int t0 = row0 + c * a.chunk_len, t1 = min(row1, t0 + a.chunk_len);
-            for (int t = t0; t < t1; ++t) decay *= a.aw[(size_t)t * 2 * a.heads + head];
-        }
+        // S_start of the chunk, and N as the start of the sums
 #pragma unroll
         for (int n = 0; n < CARRY_MAX; ++n) {
             const int e = threadIdx.x + n * 256;
             if (e >= n_elem) break;
-            const int i = e / CARRY_COLS, jj = e % CARRY_COLS, j = cb * CARRY_COLS + jj;
+            const int i = e / CARRY_COLS, j = cb * CARRY_COLS + e % CARRY_COLS;
             const float s = carry_lds[e];
             if (j < a.value_dim) ws[(size_t)i * a.ws_cols + s_off + j] = s;
-            float acc = j < a.value_dim ? ws[(size_t)i * a.ws_cols + j] : 0.f;
-            if (a.rule == 0) {
-                acc += decay * s;
-            } else {
-                const float* m = ws + (size_t)i * a.ws_cols + a.value_dim;
-                for (int k = 0; k < a.key_dim; ++k) acc += m[k] * carry_lds[k * CARRY_COLS + jj];
+            next[n] = j < a.value_dim ? ws[(size_t)i * a.ws_cols + j] : 0.f;
+            if (a.rule == 0) next[n] += decays[c] * s;
+        }
+        if (a.rule == 1) {
+#pragma unroll
+            for (int n = 0; n < CARRY_MAX; ++n) {
+                const int e = threadIdx.x + n * 256;
+                if (e >= n_elem) break;
+                const int i = e / CARRY_COLS, jj = e % CARRY_COLS;
+                const float* m = ws + (size_t)i * a.ws_cols + a.value_dim;      // row i of M: the threads of a row read it together
+                float acc0 = 0.f, acc1 = 0.f;
+                int k = 0;
+                for (; k + 1 < a.key_dim; k += 2) {
+                    acc0 += m[k] * carry_lds[k * CARRY_COLS + jj];
+                    acc1 += m[k + 1] * carry_lds[(k + 1) * CARRY_COLS + jj];
+                }
+                if (k < a.key_dim) acc0 += m[k] * carry_lds[k * CARRY_COLS + jj];
+                next[n] += acc0 + acc1;
             }
-            next[n] = acc;
         }
         __syncthreads();
 #pragma unroll
@@ -531,7 +553,7 @@ extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
     s.ws_cols = 2 * vd + (a->rule == 1 ? kd : 0);
     s.chunk_len = SCAN_CHUNK_TOKENS;
     auto ws_floats = [&]() { return (size_t)v->n_seq * ceil_div(most_new, s.chunk_len) * heads * kd * s.ws_cols; };
-    while (ws_floats() > SCAN_WS_LIMIT_FLOATS && s.chunk_len < most_new) s.chunk_len *= 2;
+    while ((ws_floats() > SCAN_WS_LIMIT_FLOATS || ceil_div(most_new, s.chunk_len) > 2048) && s.chunk_len < most_new) s.chunk_len *= 2;
     s.chunks_per_seq = ceil_div(most_new, s.chunk_len);
     if (s.chunks_per_seq < 2) return launch(v->n_seq, vd);
     if (scan_workspace(ws_floats(), &s.ws)) return -1;
@@ -540,7 +562,9 @@ extern "C" int picolm_call_state_scan(void* user, const picolm_step_view* v) {
     if (launch(v->n_seq * s.chunks_per_seq, s.ws_cols - vd)) return -1;
     const int64_t carry_blocks = (int64_t)v->n_seq * heads * ceil_div(vd, CARRY_COLS);
     PICOLM_REQUIRE(carry_blocks < (1ll << 31), "state_scan: %lld workgroups exceed the grid", (long long)carry_blocks);
-    scan_carry_kernel<<<(unsigned)carry_blocks, 256, sizeof(float) * kd * CARRY_COLS, v->stream>>>(s);
+    const size_t carry_lds = sizeof(float) * ((size_t)kd * CARRY_COLS + s.chunks_per_seq);
+    PICOLM_REQUIRE(carry_lds <= 64 * 1024, "state_scan: %d chunks a sequence need %zu bytes of LDS", s.chunks_per_seq, carry_lds);
+    scan_carry_kernel<<<(unsigned)carry_blocks, 256, carry_lds, v->stream>>>(s);
     PICOLM_LAUNCH_CHECK("state_scan (carry)");
     s.mode = 3;
     return launch(v->n_seq * s.chunks_per_seq, vd);
