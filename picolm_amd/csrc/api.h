@@ -110,8 +110,8 @@ int picolm_linear(const void* A, int a_dt, const void* W, int w_dt, void* C, int
 int picolm_kv_page_order(int dt, int d, int32_t* k_idx, int32_t* v_idx);
 // What the vector-ALU attention kernels take beside keys, values and a scale (all optional: zero
 // or null is "none"): values of a size of their own, a bias by distance added to the scaled score
-// (bias[head][min(n, bias_rows - 1)] for a key n positions back), a sink (exp(sink[head]) joins the
-// softmax's denominator once, with no key and no value), and a gate (the output of head h is
+// (bias[head][min(n, bias_rows - 1)] for a key n positions back), a sink (exp(sink[head]) is one more term
+// of the softmax's denominator and adds nothing to the numerator), and a gate (the output of head h is
 // multiplied by sigmoid(gate[token * gate_stride + h * v_head_dim + c]), float rows).
 typedef struct {
     int32_t v_head_dim;

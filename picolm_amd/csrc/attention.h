@@ -45,7 +45,7 @@ struct AttnArgs {
     int dv;                     // size of a value where it is not that of a key: out and partial rows are [H][dv]
     const float* bias;          // [H][bias_rows]: added to the scaled score of a key n positions back, entry min(n, bias_rows - 1)
     int bias_rows;
-    const float* sink;          // [H]: exp(sink) joins the softmax's denominator once, with no key and no value
+    const float* sink;          // [H]: exp(sink) is one more term of the softmax's denominator; the numerator gets nothing
     const float* gate;          // float rows: the output of head h is multiplied by sigmoid(gate[token * gate_stride + h * dv + c])
     int gate_stride;
 };

@@ -1,7 +1,7 @@
 """The Begopel decoder as a list of parts, and its entry in the architecture registry.
 
-A scaled embedding; pre-norm layers (norms with weights stored around zero) whose mixer is either
-two branches side by side, a softmax attention with a sink and a gated delta rule, or a Mamba-2
+A scaled embedding; pre-norm layers (norms whose weights are offsets from one) whose mixer is either
+two branches on one input, a softmax attention with a sink and a gated delta rule, or a Mamba-2
 state-space layer, each followed by a feed-forward with a squared relu (or none); a stretch of
 layers that runs several times in a row with the same weights, every pass entered through a
 product over [x ; embedding output] and with a cache entry of its own per layer; a head tied to

@@ -1,4 +1,4 @@
-"""Two mixers side by side on the same input: each branch's output is RMS-normed over the model
+"""Two mixers as branches of one input: each branch's output is RMS-normed over the model
 width with a weight of its own, and the mean of the two joins the residual rows:
     x += 1/2 (rms(left(h)) w_left + rms(right(h)) w_right)
 One branch may ask for keys and values, the other for state; the layer call's cache entry and

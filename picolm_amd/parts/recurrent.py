@@ -5,14 +5,14 @@ when a sequence starts.
 
 GatedDeltaRule, per head with key head floor(h / (heads / key_heads)):
     q, k, v = silu(conv(W h));  q <- q / |q| / sqrt(key_dim),  k <- k / |k|
-    S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          (the read-out sees the write)
+    S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          (o is read after the update)
     a = exp(-exp(A_log) softplus(W_a h + dt_bias)),  beta = sigmoid(W_b h)
     out = W_o (rms(o) w_norm silu(W_g h))                                 rms per head
 
 Mamba2 (state-space duality), W_in h = [z | x | B | C | dt]:
     x, B, C = silu(conv([x | B | C]) + b);  dt <- softplus(dt + dt_bias)
     S <- exp(-exp(A_log) dt) S + dt B x^T;  y = S^T C + D x
-    out = W_o (rms_parts(y silu(z)) w_norm)                               the gate comes before the norm
+    out = W_o (rms_parts(y silu(z)) w_norm)                               gated first, then normed
 """
 from __future__ import annotations
 

@@ -4,7 +4,7 @@ values may have a size of their own, and the heads are gated before the output p
 
     q, k, v, g = W h;  q <- rms(q) w_q,  k <- rms(k) w_k               per head, over the head's size
     s_ij = scale (q_i . k_j) + rel[bucket(i - j)][head]                j <= i
-    p_ij = exp(s_ij) / (exp(sink_head) + sum_j' exp(s_ij'))            the sink has no key and no value
+    p_ij = exp(s_ij) / (exp(sink_head) + sum_j' exp(s_ij'))            the sink is a term of the denominator only
     out  = W_o (concat_heads(sum_j p_ij v_j) * sigmoid(g))
 
 The bias table has B rows: one per distance below B/2, then rows spaced evenly in the logarithm of

@@ -112,7 +112,7 @@ def make_weights(cfg: dict, seed: int) -> dict:
         if name == "embed":
             t = randn(*shape)
         elif last in ("norm1", "norm2") or name == "final.norm":
-            t = 0.2 * randn(*shape)                                  # stored around zero
+            t = 0.2 * randn(*shape)                                  # the norm adds one
         elif name.endswith(("q.norm", "k.norm", "left.out", "right.out", ".norm")):
             t = 1.0 + 0.2 * randn(*shape)
         elif last == "rel":

@@ -37,7 +37,7 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
 
 
 def short_conv(x, w, bias=None):
-    """x [T, C], w [C, taps]: y[t, c] = sum_j w[c, taps-1-j] x[t-j, c], zeros before the start."""
+    """x [T, C], w [C, taps]: y[t, c] = sum_j w[c, taps-1-j] x[t-j, c], with x[t] = 0 for t < 0."""
     T, C = x.shape
     taps = w.shape[1]
     y = torch.zeros_like(x)

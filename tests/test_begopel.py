@@ -115,7 +115,7 @@ def test_plain_attention_special_cases():
 
 def test_plain_short_convolution_and_bucket():
     x = torch.arange(12, dtype=torch.float64).view(6, 2)
-    w = torch.tensor([[1.0, 10.0, 100.0], [0.0, 0.0, 1.0]], dtype=torch.float64)       # the last column is the current token's
+    w = torch.tensor([[1.0, 10.0, 100.0], [0.0, 0.0, 1.0]], dtype=torch.float64)       # column taps-1 multiplies x[t]
     y = P.short_conv(x, w)
     assert y[:, 1].tolist() == x[:, 1].tolist()
     assert y[0, 0] == 0.0 and y[1, 0] == 100.0 * 2 + 10.0 * 0 and y[3, 0] == 100.0 * 6 + 10.0 * 4 + 1.0 * 2
