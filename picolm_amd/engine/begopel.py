@@ -10,13 +10,14 @@ from __future__ import annotations
 
 from ..config import register_architecture
 from ..config.begopel import BegopelConfig, Mamba2Config, ParallelConfig
-from ..parts import LMHead, PreNormBlock, RMSNorm, TokenEmbedding
+from ..parts import LMHead, Part, PreNormBlock, RMSNorm, TokenEmbedding
 from ..parts.block import LoopEntry
 from ..parts.feedforward import ActivatedMLP
 from ..parts.linear import Linear
 from ..parts.parallel import ParallelMixer
 from ..parts.recurrent import GatedDeltaRule, Mamba2
 from ..parts.sink_attention import SinkAttention
+from ..weights import TensorSpec
 from .model import DecoderModel, LayerCall
 
 
@@ -32,6 +33,17 @@ def _mixer(prefix: str, kind, D: int, eps: float):
     raise ValueError(f"no mixer for {type(kind).__name__}")
 
 
+class _UnusedTensors(Part):
+    """Tensors that a checkpoint may carry and the model never reads (the second norm of a layer
+    that has no feed-forward): named, so that the check of the checkpoint passes them by."""
+
+    def __init__(self, specs):
+        self._specs = list(specs)
+
+    def tensor_specs(self):
+        return self._specs
+
+
 def build_begopel(cfg: BegopelConfig) -> DecoderModel:
     D, eps = cfg.width, cfg.norm_eps
     blocks = []
@@ -43,6 +55,8 @@ def build_begopel(cfg: BegopelConfig) -> DecoderModel:
                                    ActivatedMLP(p + "mlp.", D, layer.ff, "relu_squared") if has_ff else None))
     n_layers = len(blocks)
     order = []
+    unused = _UnusedTensors(TensorSpec(f"l{i}.norm2", (D,), optional=True, init=None)
+                            for i, layer in enumerate(cfg.layers) if layer.ff is None)
     if cfg.loop is not None:
         w_in = Linear(["loop.in"], [D], 2 * D)
         blocks += [LoopEntry(w_in, "loop.step", D, cfg.loop.times, t) for t in range(cfg.loop.times)]
@@ -51,8 +65,10 @@ def build_begopel(cfg: BegopelConfig) -> DecoderModel:
             order.append(LayerCall(n_layers + t))
         order.append(LayerCall(i))
     emb = TokenEmbedding("embed", cfg.vocab, D, scale=cfg.embedding_scale, keeps_output=cfg.loop is not None)
-    return DecoderModel(cfg, emb, blocks, RMSNorm("final.norm", D, eps, weight_offset=1.0),
-                        LMHead("lm_head", cfg.vocab, D, emb, tied=True, softcap=cfg.logit_softcap), order)
+    model = DecoderModel(cfg, emb, blocks, RMSNorm("final.norm", D, eps, weight_offset=1.0),
+                         LMHead("lm_head", cfg.vocab, D, emb, tied=True, softcap=cfg.logit_softcap), order)
+    model.extra_parts = [unused]
+    return model
 
 
 register_architecture("Begopel", BegopelConfig.from_dict, build_begopel, replace=True)

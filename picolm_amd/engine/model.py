@@ -42,11 +42,12 @@ class DecoderModel:
             if c.reads_cache_of is not None and not 0 <= c.reads_cache_of < i:
                 raise ValueError(f"layer call {i} can only read the cache of an earlier call")
         self.runtime: Runtime | None = None
+        self.extra_parts: list = []         # parts outside the layers: they declare and load tensors, and emit nothing
         self._plan_cache()
 
     # -- structure --------------------------------------------------------------------------
     def parts(self):
-        return [self.embedding, *self.blocks, self.final_norm, self.head]
+        return [self.embedding, *self.blocks, self.final_norm, self.head, *self.extra_parts]
 
     def tensor_specs(self):
         out, seen = [], set()

@@ -150,3 +150,21 @@ def test_plain_delta_rule_and_state_space_recurrences():
     v = P.silu(h[:, 1:3])
     want = P.rms(v * 2 ** -0.5, 0.0) * 40.0     # the read-out is v times the query's length 1/sqrt(dim)
     assert torch.allclose(out, want, rtol=1e-6)
+
+
+def test_an_unused_second_norm_is_passed_by_and_a_stray_tensor_is_not():
+    from picolm_amd.engine.builder import build_from_config_dict
+    from picolm_amd.weights import TensorDict, WeightsError, check_specs
+    cfg = bt.config(61, 48, [bt.mamba(2, 8, 8, 1, 1, 2, None)])
+    w = bt.make_weights(cfg, 0)
+    specs = build_from_config_dict(cfg).tensor_specs()
+    check_specs(TensorDict(w), specs)
+    check_specs(TensorDict({**w, "l0.norm2": torch.zeros(48, dtype=torch.bfloat16)}), specs)
+    with pytest.raises(WeightsError) as e:
+        check_specs(TensorDict({**w, "l0.norm3": torch.zeros(48, dtype=torch.bfloat16)}), specs)
+    assert "l0.norm3" in str(e.value)
+    # the distance table's rows are the tensor's to say where the configuration does not name them
+    cfg = bt.config(61, 48, [bt.parallel(bt.attention(2, 1, 8, 8, 0.3, 9.0, 4), bt.delta(2, 1, 8, 8, 2), None)])
+    w = bt.make_weights(cfg, 0)
+    del cfg["layers"][0]["mixer"]["left"]["bias_rows"]
+    check_specs(TensorDict(w), build_from_config_dict(cfg).tensor_specs())
