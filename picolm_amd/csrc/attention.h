@@ -48,6 +48,10 @@ struct AttnArgs {
     const float* sink;          // [H]: exp(sink) is one more term of the softmax's denominator; the numerator gets nothing
     const float* gate;          // float rows: the output of head h is multiplied by sigmoid(gate[token * gate_stride + h * dv + c])
     int gate_stride;
+    // attention_plain_mfma.hip, prefill: the waves of a workgroup take adjacent query heads (of one KV
+    // group) over all keys, so that they read the same keys and values at about the same time;
+    // zero: they take one head's keys in turn
+    int waves_take_heads;
 };
 
 // ---- the order of a page's elements ---------------------------------------------------------

@@ -1,18 +1,22 @@
-// bf16 softmax attention on the matrix cores over pages kept as plain arrays (K[64][d],
-// V^T[dv][64]), with what the vector-ALU kernels of attention_generic.hip take beside keys and
+// bf16 softmax attention on the matrix cores over pages that the caller keeps in the order of the
+// MFMA operands (attention.h: k_page_offset(key, i, d, true), v_page_offset(i, key, dv, true)), with what the vector-ALU kernels of attention_generic.hip take beside keys and
 // values: values of a size of their own, a bias by distance, a sink and an output gate.  Head sizes
 // of 64, 96 and 128 on either side.
 //
-// One wave per piece of work, no LDS: S^T = K Q^T and O^T = V^T P^T with 32x32x16 MFMAs as in
+// A workgroup of PLAIN_WAVES waves per piece of work; the waves take the tiles of 32 keys in turn and
+// add their results up through LDS at the end.  S^T = K Q^T and O^T = V^T P^T with 32x32x16 MFMAs as in
 // attention_mfma.hip (a lane of the accumulator holds one query and 16 keys, so the softmax's
 // maximum and sum are in-lane plus one exchange with lane ^ 32, and P^T feeds the second product
-// from registers).  A lane's operand of K is 16 bytes of one key's row, of V^T 16 bytes of one
-// value column's row: the rows of a tile are read whole over the k-steps, through the caches.
-//   prefill: a wave takes 32 new tokens of one head (the step's tiles of 32 rows) and walks the
-//            keys it sees, 32 at a time; the next tile's operands are asked for before this
-//            tile's products.
-//   decode : a wave takes one entry of the step's work list and one KV group; its columns are the
-//            group's query heads (32 at a time).  A sequence of several chunks leaves partial
+// from registers).  (Pages as plain arrays were measured first: a lane's 16 bytes of a key's row
+// lie in a cache line of their own, a tile cost a thousand line look-ups in the CU's cache, and a
+// tile took 8 us.)
+//   prefill: a workgroup takes 32 new tokens (the step's tiles of 32 rows): of four query heads of one
+//            KV group where the group has a multiple of four, a head a wave, so that the waves read
+//            the same keys and values at about the same time and three of them find them in the
+//            CU's cache; else of one head, whose keys the waves take in turn, 32 at a time; a wave's next tile's operands are asked for before
+//            this tile's products, and the page after that is looked up in the page table.
+//   decode : a workgroup takes one entry of the step's work list and one KV group; its columns are
+//            the group's query heads (32 at a time).  A sequence of several chunks leaves partial
 //            results for the merge kernel of attention_generic.hip.
 // Statistics are float in the base-2 domain; the bias table is [H][bias_rows].
 #include "common.h"
@@ -35,22 +39,27 @@ struct TileOperands {
     bf16x8 V[DV / 32][2];
 };
 
-// operands of the 32 keys from key `half * 32` of a page on
+// operands of the 32 keys from key `half * 32` of a page on: the pages are in the order of the
+// operands (k_page_offset, v_page_offset of attention.h, the values' rows counted by DV), so that a
+// wave's load of a chunk reads 1 KB in a row
 template <int D, int DV>
-__device__ __forceinline__ void load_tile(TileOperands<D, DV>& t, const bf16_t* kpage, const bf16_t* vpage, int half, int col, int h) {
-    const bf16_t* kp = kpage + (size_t)(32 * half + key_of_row(col)) * D + 8 * h;
+__device__ __forceinline__ void load_tile(TileOperands<D, DV>& t, const bf16_t* kpage, const bf16_t* vpage, int half, int lane) {
+    const bf16_t* kp = kpage + ((size_t)half * (D / 16) * 64 + lane) * 8;
 #pragma unroll
-    for (int s = 0; s < D / 16; ++s) t.K[s] = ldg8(kp + 16 * s);
-    const bf16_t* vp = vpage + (size_t)col * PAGE_TOKENS + 32 * half + 8 * h;
+    for (int s = 0; s < D / 16; ++s) t.K[s] = ldg8(kp + 512 * s);
+    const bf16_t* vp = vpage + ((size_t)half * (DV / 32) * 2 * 64 + lane) * 8;
 #pragma unroll
     for (int dt = 0; dt < DV / 32; ++dt)
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) t.V[dt][ks] = ldg8(vp + (size_t)32 * dt * PAGE_TOKENS + 16 * ks);
+        for (int ks = 0; ks < 2; ++ks) t.V[dt][ks] = ldg8(vp + 512 * (2 * dt + ks));
 }
 
+#define PLAIN_WAVES 4
+
 template <int D, int DV>
-__global__ __launch_bounds__(64) void attn_plain_mfma_kernel(AttnArgs a) {
-    const int lane = threadIdx.x, col = lane & 31, h = lane >> 5;
+__global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_plain_mfma_kernel(AttnArgs a) {
+    extern __shared__ float merge_lds[];        // [PLAIN_WAVES - 1][DV / 2 + 2][64]: O^T, maximum and sum of the other waves
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, col = lane & 31, h = lane >> 5;
     const int R = a.H / a.G;
     int seq, g, head, tok, qpos, qpos_first, slot, page_lo, page_hi, hi, split = 0, n_chunks = 1;
     bool q_ok;
@@ -69,7 +78,7 @@ __global__ __launch_bounds__(64) void attn_plain_mfma_kernel(AttnArgs a) {
     } else {
         seq = a.tile_seq[blockIdx.x];
         const int q0 = a.tile_q0[blockIdx.x], nnew = a.seq_nnew[seq], pos0 = a.seq_pos0[seq];
-        head = blockIdx.y;
+        head = a.waves_take_heads ? blockIdx.y * PLAIN_WAVES + wave : blockIdx.y;
         g = head / R;
         q_ok = q0 + col < nnew;
         const int l = min(q0 + col, nnew - 1);
@@ -101,33 +110,47 @@ __global__ __launch_bounds__(64) void attn_plain_mfma_kernel(AttnArgs a) {
     const bf16_t* vbase = (const bf16_t*)a.v_pages + (size_t)g * PAGE_TOKENS * DV;
     const size_t k_page_elems = (size_t)a.G * PAGE_TOKENS * D, v_page_elems = (size_t)a.G * PAGE_TOKENS * DV;
 
-    const int tile_lo = 2 * page_lo, tile_hi = min(2 * page_hi, hi / 32 + 1);       // tiles of 32 keys: [tile_lo, tile_hi)
-    TileOperands<D, DV> cur, nxt;
-    if (tile_lo < tile_hi) {
-        const int phys = pt[(tile_lo / 2) % a.ring_pages];
-        load_tile<D, DV>(cur, kbase + (size_t)phys * k_page_elems, vbase + (size_t)phys * v_page_elems, tile_lo & 1, col, h);
-    }
-    for (int t = tile_lo; t < tile_hi; ++t) {
-        if (t + 1 < tile_hi) {
-            const int phys = pt[((t + 1) / 2) % a.ring_pages];
-            load_tile<D, DV>(nxt, kbase + (size_t)phys * k_page_elems, vbase + (size_t)phys * v_page_elems, (t + 1) & 1, col, h);
+    const int tile_hi = min(2 * page_hi, hi / 32 + 1);       // tiles of 32 keys: this wave takes tile_lo, tile_lo + PLAIN_WAVES, ... below tile_hi
+    const bool keys_in_turn = !a.waves_take_heads;           // the waves share one head's keys
+    const int tile_step = keys_in_turn ? PLAIN_WAVES : 1;
+    const int tile_lo = 2 * page_lo + (keys_in_turn ? wave : 0);
+    // two sets of operands in turn: the loads of the tile after this one are queued before this
+    // tile's products and stay there (the scheduler may not move them past the barrier), and the
+    // page of the tile after that is looked up meanwhile
+    TileOperands<D, DV> A, B;
+    auto fetch = [&](TileOperands<D, DV>& ops, int t, int phys) {
+        load_tile<D, DV>(ops, kbase + (size_t)phys * k_page_elems, vbase + (size_t)phys * v_page_elems, t & 1, lane);
+    };
+    auto page_of = [&](int t) { return t < tile_hi ? pt[(t / 2) % a.ring_pages] : 0; };
+    // a tile's 16 biases of a lane, in base-2 units: asked for before the next tile's operands, because
+    // loads come back in the order they were queued and the softmax must not wait for those too
+    auto load_bias = [&](int t, float (&bv)[16]) {
+        const int key0 = 32 * t;
+        if (!bias || t >= tile_hi) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) bv[e] = 0.f;
+        } else if (qpos_first - (key0 + 31) >= last_row) {      // wave-uniform: every pair of the tile is beyond the table
+            const float far_bias = bias[last_row] * LOG2E;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) bv[e] = far_bias;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) bv[e] = bias[min(max(qpos - (key0 + key_of_elem(e, h)), 0), last_row)] * LOG2E;
         }
+    };
+    auto attend = [&](const TileOperands<D, DV>& ops, int t, const float (&bv)[16]) {
         const int key0 = 32 * t;
         f32x16 S;
 #pragma unroll
         for (int e = 0; e < 16; ++e) S[e] = 0.f;
 #pragma unroll
-        for (int s = 0; s < D / 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.K[s], Qf[s], S, 0, 0, 0);
-        const bool far = bias && qpos_first - (key0 + 31) >= last_row;       // wave-uniform: every pair of the tile is beyond the table
-        const float far_bias = bias ? bias[last_row] * LOG2E : 0.f;
+        for (int s = 0; s < D / 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.K[s], Qf[s], S, 0, 0, 0);
         float mx = NEG_BIG;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int key = key0 + key_of_elem(e, h);
             const bool vis = q_ok && key <= qpos;
-            float s2 = S[e] * scale2;
-            if (bias) s2 += far ? far_bias : bias[min(max(qpos - key, 0), last_row)] * LOG2E;
-            S[e] = vis ? s2 : NEG_BIG;
+            S[e] = vis ? fmaf(S[e], scale2, bv[e]) : NEG_BIG;
             mx = fmaxf(mx, S[e]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
@@ -149,9 +172,55 @@ __global__ __launch_bounds__(64) void attn_plain_mfma_kernel(AttnArgs a) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) O[dt][e] *= alpha;
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur.V[dt][ks], Pf[ks], O[dt], 0, 0, 0);
+            for (int ks = 0; ks < 2; ++ks) O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ops.V[dt][ks], Pf[ks], O[dt], 0, 0, 0);
         }
-        cur = nxt;
+    };
+    if (tile_lo < tile_hi) fetch(A, tile_lo, page_of(tile_lo));
+    int phys_b = page_of(tile_lo + tile_step), phys_a = 0;
+    float bv[16];
+    for (int t = tile_lo; t < tile_hi; t += 2 * tile_step) {
+        const int tb = t + tile_step, ta = t + 2 * tile_step;
+        load_bias(t, bv);
+        __builtin_amdgcn_sched_barrier(0);
+        if (tb < tile_hi) fetch(B, tb, phys_b);
+        phys_a = page_of(ta);
+        __builtin_amdgcn_sched_barrier(0);
+        attend(A, t, bv);
+        if (tb >= tile_hi) break;
+        load_bias(tb, bv);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ta < tile_hi) fetch(A, ta, phys_a);
+        phys_b = page_of(ta + tile_step);
+        __builtin_amdgcn_sched_barrier(0);
+        attend(B, tb, bv);
+    }
+    // the other waves' results join the first wave's
+    if (PLAIN_WAVES > 1 && keys_in_turn) {
+        constexpr int PER = DV / 2 + 2;          // floats a lane leaves
+        if (wave > 0) {
+            float* mine = merge_lds + (size_t)(wave - 1) * PER * 64 + lane;
+            mine[0] = m_run;
+            mine[64] = l_run;
+#pragma unroll
+            for (int dt = 0; dt < DV / 32; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mine[(2 + 16 * dt + e) * 64] = O[dt][e];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 0; w < PLAIN_WAVES - 1; ++w) {
+            const float* other = merge_lds + (size_t)w * PER * 64 + lane;
+            const float m_o = other[0], l_o = other[64];
+            const float m_new = fmaxf(m_run, m_o);
+            const float mine_k = exp2_flushing(m_run - m_new), other_k = exp2_flushing(m_o - m_new);
+            l_run = l_run * mine_k + l_o * other_k;
+            m_run = m_new;
+#pragma unroll
+            for (int dt = 0; dt < DV / 32; ++dt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) O[dt][e] = O[dt][e] * mine_k + other[(2 + 16 * dt + e) * 64] * other_k;
+        }
     }
     if (!q_ok) return;
     // element 4 a + b of O[dt] is value column 32 dt + 8 a + 4 h + b of query `col`
@@ -194,9 +263,10 @@ extern "C" int picolm_attn_plain_mfma_tile_rows(void) { return 32; }
 
 template <int D>
 static int launch_dv(const AttnArgs& a, int dv, dim3 grid, hipStream_t stream) {
-    if (dv == 64) attn_plain_mfma_kernel<D, 64><<<grid, 64, 0, stream>>>(a);
-    else if (dv == 96) attn_plain_mfma_kernel<D, 96><<<grid, 64, 0, stream>>>(a);
-    else attn_plain_mfma_kernel<D, 128><<<grid, 64, 0, stream>>>(a);
+    const size_t lds = sizeof(float) * (PLAIN_WAVES - 1) * (dv / 2 + 2) * 64;       // at most 50 KB
+    if (dv == 64) attn_plain_mfma_kernel<D, 64><<<grid, 64 * PLAIN_WAVES, lds, stream>>>(a);
+    else if (dv == 96) attn_plain_mfma_kernel<D, 96><<<grid, 64 * PLAIN_WAVES, lds, stream>>>(a);
+    else attn_plain_mfma_kernel<D, 128><<<grid, 64 * PLAIN_WAVES, lds, stream>>>(a);
     PICOLM_LAUNCH_CHECK("attn_plain_mfma");
     return 0;
 }
@@ -233,7 +303,10 @@ extern "C" int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages
                   nullptr, nullptr, nullptr, nullptr, 0};
     int dv;
     if (fill_extras("attn_prefill_plain_mfma", a, x, dv)) return -1;
-    return launch(a, dv, dim3(n_tiles, H), stream);
+    // (measured at 2,048 tokens: a head a wave is faster once its workgroups fill the 256 CUs, 0.39 against 0.47 ms
+    // for two layers of 16 heads; with 8 heads the keys in turn are, 0.40 against 0.57 ms)
+    a.waves_take_heads = (H / G) % PLAIN_WAVES == 0 && (int64_t)n_tiles * (H / PLAIN_WAVES) >= 256;
+    return launch(a, dv, dim3(n_tiles, a.waves_take_heads ? H / PLAIN_WAVES : H), stream);
 }
 
 extern "C" int picolm_attn_decode_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, int n_seq,

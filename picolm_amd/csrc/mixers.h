@@ -32,7 +32,8 @@ int picolm_call_loop_input(void* user, const picolm_step_view* v);
 //   [H d] in the engine's dtype.  Flags: PICOLM_CALL_KV | PICOLM_CALL_ATTENDS, partial_floats =
 //   H (dv + 2), tile_rows = picolm_attn_plain_mfma_tile_rows() where the engine runs in bfloat16 and
 //   picolm_attn_plain_mfma_takes(d, dv) (the matrix-core kernel then runs), else
-//   picolm_attn_prefill_tile_rows().  Pages are kept as plain arrays.
+//   picolm_attn_prefill_tile_rows().  The operation writes its own pages: as plain arrays, or for the
+//   matrix-core kernel in the order of its operands.
 typedef struct {
     int32_t n_heads, n_kv_heads, head_dim, v_head_dim;
     int32_t in_stride, q_off, k_off, v_off, gate_off;     // gate_off < 0: no gate

@@ -9,6 +9,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "attention.h"
 
 #define VIEW_REQUIRE(who, v)                                                                                      \
     PICOLM_REQUIRE((v) && (v)->struct_bytes == (int32_t)sizeof(picolm_step_view), "%s: the step view is of another version", who)
@@ -49,13 +50,13 @@ extern "C" int picolm_call_loop_input(void* user, const picolm_step_view* v) {
 
 // ---- attention with a norm of queries and keys, a bias by distance, a sink and a gate ------------
 // One wave per (token, head): query heads go, normed, to the rows the attention kernel reads;
-// key heads, normed, and value heads to the token's place in its cache page (plain arrays
-// K[G][64][d], V^T[G][dv][64]).
+// key heads, normed, and value heads to the token's place in its cache page (K[G][64][d],
+// V^T[G][dv][64] as plain arrays, or with `tiled` in the order of the MFMA operands).
 template <typename T>
 __global__ void qk_norm_store_kernel(const float* __restrict__ in, int in_stride, int q_off, int k_off, int v_off, T* __restrict__ q_out,
                                      T* __restrict__ k_pages, T* __restrict__ v_pages, const float* __restrict__ q_norm,
                                      const float* __restrict__ k_norm, float eps, const int32_t* __restrict__ tok_pos,
-                                     const int32_t* __restrict__ write_pages, int H, int G, int d, int dv) {
+                                     const int32_t* __restrict__ write_pages, int H, int G, int d, int dv, bool tiled) {
     const size_t row = blockIdx.x;
     const int unit = blockIdx.y, lane = threadIdx.x;
     const float* src = in + row * in_stride;
@@ -71,20 +72,20 @@ __global__ void qk_norm_store_kernel(const float* __restrict__ in, int in_stride
             ssq = wave_sum(ssq);
             inv = 1.f / sqrtf(ssq / (float)d + eps);
         }
-        T* dst;
         if (is_q) {
-            dst = q_out + (row * H + head) * d;
+            T* dst = q_out + (row * H + head) * d;
+            for (int i = lane; i < d; i += WAVE) dst[i] = from_f32<T>(w ? x[i] * inv * w[i] : x[i]);
         } else {
             const int key = tok_pos[row] % PAGE_TOKENS;
-            dst = k_pages + ((size_t)write_pages[row] * G + head) * PAGE_TOKENS * d + (size_t)key * d;
+            T* dst = k_pages + ((size_t)write_pages[row] * G + head) * PAGE_TOKENS * d;
+            for (int i = lane; i < d; i += WAVE) dst[k_page_offset(key, i, d, tiled)] = from_f32<T>(w ? x[i] * inv * w[i] : x[i]);
         }
-        for (int i = lane; i < d; i += WAVE) dst[i] = from_f32<T>(w ? x[i] * inv * w[i] : x[i]);
     } else {
         const int head = unit - H - G;
         const float* x = src + v_off + (size_t)head * dv;
         const int key = tok_pos[row] % PAGE_TOKENS;
-        T* dst = v_pages + ((size_t)write_pages[row] * G + head) * dv * PAGE_TOKENS + key;
-        for (int i = lane; i < dv; i += WAVE) dst[(size_t)i * PAGE_TOKENS] = from_f32<T>(x[i]);
+        T* dst = v_pages + ((size_t)write_pages[row] * G + head) * dv * PAGE_TOKENS;
+        for (int i = lane; i < dv; i += WAVE) dst[v_page_offset(i, key, dv, tiled)] = from_f32<T>(x[i]);
     }
 }
 
@@ -108,14 +109,15 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     if (v->n_tokens <= 0) return 0;
     const float* in = (const float*)v->in;
     dim3 grid(v->n_tokens, v->kv_writes ? H + 2 * G : H);
+    const bool mfma = dt == PICOLM_BF16 && picolm_attn_plain_mfma_takes(d, dv);      // then the pages are in the matrix-core kernel's order
     if (dt == PICOLM_F32)
         qk_norm_store_kernel<float><<<grid, WAVE, 0, v->stream>>>(in, a->in_stride, a->q_off, a->k_off, a->v_off, (float*)v->extra[0],
                                                                   (float*)v->k_pages, (float*)v->v_pages, a->q_norm, a->k_norm, a->eps,
-                                                                  v->tok_pos, v->write_pages, H, G, d, dv);
+                                                                  v->tok_pos, v->write_pages, H, G, d, dv, false);
     else
         qk_norm_store_kernel<bf16_t><<<grid, WAVE, 0, v->stream>>>(in, a->in_stride, a->q_off, a->k_off, a->v_off, (bf16_t*)v->extra[0],
                                                                    (bf16_t*)v->k_pages, (bf16_t*)v->v_pages, a->q_norm, a->k_norm, a->eps,
-                                                                   v->tok_pos, v->write_pages, H, G, d, dv);
+                                                                   v->tok_pos, v->write_pages, H, G, d, dv, mfma);
     PICOLM_LAUNCH_CHECK("sink_attention (norm and cache write)");
     picolm_attn_extras x;
     x.v_head_dim = dv;
@@ -124,7 +126,6 @@ extern "C" int picolm_call_sink_attention(void* user, const picolm_step_view* v)
     x.sink = a->sink;
     x.gate = a->gate_off >= 0 ? in + a->gate_off : nullptr;
     x.gate_stride = a->in_stride;
-    const bool mfma = dt == PICOLM_BF16 && picolm_attn_plain_mfma_takes(d, dv);
     if (mfma && v->is_decode)
         return picolm_attn_decode_plain_mfma(v->extra[0], v->k_pages, v->v_pages, v->out, v->partial, v->n_seq, v->chunk_list, v->n_chunks,
                                              v->pages_per_chunk, v->most_chunks, v->seq_pos0, v->page_table, v->max_pages, v->ring_pages, H,
