@@ -604,7 +604,7 @@ __global__ void gated_norm_kernel(const float* __restrict__ x, const float* __re
 
 // the same with a workgroup per (row, part), for parts of a thousand columns and more
 template <typename T>
-__global__ __launch_bounds__(256) void gated_norm_wide_kernel(const float* __restrict__ x, const float* __restrict__ gate, int gate_stride,
+__global__ __launch_bounds__(1024) void gated_norm_wide_kernel(const float* __restrict__ x, const float* __restrict__ gate, int gate_stride,
                                                               int gate_off, T* __restrict__ out, const float* __restrict__ weight,
                                                               int weight_len, int width, int group, float eps, int gate_first) {
     __shared__ float scratch[16];
@@ -643,12 +643,14 @@ extern "C" int picolm_call_gated_norm(void* user, const picolm_step_view* v) {
     const int64_t n_units = (int64_t)v->rows * (a->width / a->group);
     PICOLM_REQUIRE(n_units < (1ll << 31), "gated_norm: %lld workgroups exceed the grid", (long long)n_units);
     if (a->group >= 1024) {
+        // few rows (a decode step): more threads a part, so that a thread's loads, each of which it waits for, are few
+        const int threads = n_units < 1024 ? 1024 : 256;
         if (v->dtype == PICOLM_F32)
-            gated_norm_wide_kernel<float><<<(unsigned)n_units, 256, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0], a->gate_stride,
+            gated_norm_wide_kernel<float><<<(unsigned)n_units, threads, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0], a->gate_stride,
                                                                                     a->gate_off, (float*)v->out, a->weight, a->weight_len,
                                                                                     a->width, a->group, a->eps, a->gate_first);
         else
-            gated_norm_wide_kernel<bf16_t><<<(unsigned)n_units, 256, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0],
+            gated_norm_wide_kernel<bf16_t><<<(unsigned)n_units, threads, 0, v->stream>>>((const float*)v->in, (const float*)v->extra[0],
                                                                                      a->gate_stride, a->gate_off, (bf16_t*)v->out, a->weight,
                                                                                      a->weight_len, a->width, a->group, a->eps, a->gate_first);
         PICOLM_LAUNCH_CHECK("gated_norm (wide)");
@@ -668,7 +670,7 @@ extern "C" int picolm_call_gated_norm(void* user, const picolm_step_view* v) {
 }
 
 // ---- two normed branches meet the residual rows ------------------------------------------------------
-__global__ void normed_sum_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
+__global__ __launch_bounds__(1024) void normed_sum_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
                                   const float* __restrict__ w_a, const float* __restrict__ w_b, int W, float eps, float mult) {
     __shared__ float scratch[16];
     const size_t row = blockIdx.x;
@@ -700,7 +702,7 @@ extern "C" int picolm_call_normed_sum(void* user, const picolm_step_view* v) {
     PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * 4 && (!v->extra[0] || v->extra_row_bytes[0] >= a->width * 4),
                    "normed_sum: rows too short for a width of %d", a->width);
     if (v->rows <= 0) return 0;
-    normed_sum_kernel<<<v->rows, 256, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0], a->w_a, a->w_b, a->width,
+    normed_sum_kernel<<<v->rows, v->rows < 1024 && a->width >= 1024 ? 1024 : 256, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0], a->w_a, a->w_b, a->width,
                                                       a->eps, a->mult);
     PICOLM_LAUNCH_CHECK("normed_sum");
     return 0;
