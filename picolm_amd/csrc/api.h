@@ -134,7 +134,8 @@ int picolm_attn_decode_plain(const void* q, const void* k_pages, const void* v_p
                              const int32_t* page_table, int max_pages, int ring_pages, int H, int G, int d, int window, float scale,
                              const picolm_attn_extras* x, hipStream_t stream);
 // The same on the matrix cores: bfloat16, keys and values of the sizes that picolm_attn_plain_mfma_takes
-// says, prefill tiles of picolm_attn_plain_mfma_tile_rows() rows, no window.
+// says, prefill tiles of picolm_attn_plain_mfma_tile_rows() rows, no window; the caller's pages are in the
+// order of the MFMA operands (attention.h: k_page_offset(key, i, d, true), v_page_offset(i, key, dv, true)).
 int picolm_attn_plain_mfma_takes(int d, int dv);
 int picolm_attn_plain_mfma_tile_rows(void);
 int picolm_attn_prefill_plain_mfma(const void* q, const void* k_pages, const void* v_pages, void* out, const int32_t* tile_seq,
