@@ -77,9 +77,7 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold together, each rounded up to 64")
     args = ap.parse_args(argv)
     model = load_model(args.model, dtype=args.dtype)
-    # every request's tokens are held in whole pages of 64: room for a part-filled page each, for
-    # as many requests as the budget could hold a page of
-    session = Session(model, max_tokens=args.max_tokens + 64 * min(max(args.max_tokens // 64, 1), 256))
+    session = Session(model, max_tokens=args.max_tokens)
     rp = Replayer(session, args.out)
     for line in sys.stdin:
         line = line.strip()
