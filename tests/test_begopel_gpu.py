@@ -82,6 +82,10 @@ ALONE = {
     # head sizes that the matrix-core attention takes in bfloat16 (64, 96, 128 on either side), with more than 32 heads a group
     "attention, sizes of real heads": (one_layer(bt.parallel(bt.attention(4, 2, 96, 64, 0.2, 25.0, 10), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
     "attention, forty heads a group": (one_layer(bt.parallel(bt.attention(40, 1, 64, 128, 0.25, 70.0, 16), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
+    "attention, heads of 128": (one_layer(bt.parallel(bt.attention(4, 1, 128, 128, 0.1, 33.0, 12), bt.delta(2, 1, 8, 12, 2), None)), "right.out"),
+    # keys beyond 128 lie in sixteen lanes a column
+    "delta, keys of 144": (one_layer(bt.parallel(bt.attention(2, 1, 8, 8, 0.3, 9.0, 4), bt.delta(2, 1, 144, 8, 2), None)), "left.out"),
+    "mamba, a state of 200": (one_layer(bt.mamba(2, 8, 200, 1, 1, 2, None)), None),
     "mamba": (one_layer(bt.mamba(6, 8, 12, 3, 2, 3, None)), None),
     "mamba, a wide norm": (one_layer(bt.mamba(20, 64, 8, 1, 1, 2, None)), None),
     "mamba, one tap": (one_layer(bt.mamba(2, 24, 20, 1, 3, 1, None)), None),
@@ -200,6 +204,33 @@ def test_long_prompts_walked_in_chunks(which, dtype):
         assert bt.distance(got[1 + i], truth_of(which, 0, q)[-1]) <= bt.LIMIT[dtype], ("beside the long one", i)
     got = s.step(slots[:1], [[tokens[400]]]).double().cpu().numpy()
     assert bt.distance(got, want[400]) <= bt.LIMIT[dtype]
+    s.release(slots)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_prefill_step_wide_enough_for_a_head_a_wave(dtype):
+    """With four or more query heads a KV group and at least 256 workgroups of (32 queries, four
+    heads), the matrix-core attention gives each wave of a workgroup a head of its own instead of
+    a share of one head's keys: 18 prompts of 100 to 160 tokens and 16 heads over 4 groups make
+    such a step (bfloat16; the 32-bit runtime takes the vector-ALU kernel through the same test)."""
+    cfg = bt.config(83, 64, [bt.parallel(bt.attention(16, 4, 64, 64, 0.3, 90.0, 16), bt.delta(2, 1, 8, 12, 2), None)], scale=2.0)
+    w = bt.make_weights(cfg, 21)
+    w["l0.mix.right.out"] = torch.zeros_like(w["l0.mix.right.out"])
+    lens = [100 + (37 * i) % 61 for i in range(18)]
+    assert sum((n + 31) // 32 for n in lens) * (16 // 4) >= 256
+    seqs = [tokens_for(cfg, n + 2, 300 + i) for i, n in enumerate(lens)]
+    s = new_session(bt.load(cfg, w, dtype), 4096)
+    slots = s.begin(len(seqs))
+    got = s.step(slots, [q[:n] for q, n in zip(seqs, lens)], [list(range(n)) for n in lens]).double().cpu().numpy()
+    truth = [bt.plain_logits(cfg, w, q) for q in seqs]
+    at = 0
+    for i, n in enumerate(lens):
+        assert bt.distance(got[at:at + n], truth[i][:n]) <= bt.LIMIT[dtype], ("prompt", i)
+        at += n
+    for j in range(2):
+        got = s.step(slots, [[q[n + j]] for q, n in zip(seqs, lens)]).double().cpu().numpy()
+        for i, n in enumerate(lens):
+            assert bt.distance(got[i], truth[i][n + j]) <= bt.LIMIT[dtype], ("step", j, "sequence", i)
     s.release(slots)
 
 
