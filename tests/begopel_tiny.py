@@ -64,7 +64,13 @@ CONFIG_R = config(515, 256, [
     mamba(4, 64, 128, 2, 1, 4, 512),
 ], scale=16.0, eps=1e-6, softcap=30.0)
 
-CONFIGS = {"P": CONFIG_P, "Q": CONFIG_Q, "R": CONFIG_R}
+# S: no size is a multiple of 8 (width 50, heads of 10, 6, 5 and 7, three heads, three norm parts)
+CONFIG_S = config(77, 50, [
+    parallel(attention(3, 1, 10, 6, 0.3, 11.0, 5), delta(3, 1, 10, 5, 3), 33),
+    mamba(3, 5, 7, 1, 3, 3, 21),
+], loop=(0, 2, 2), scale=2.0, softcap=9.0)
+
+CONFIGS = {"P": CONFIG_P, "Q": CONFIG_Q, "R": CONFIG_R, "S": CONFIG_S}
 
 
 def tensor_shapes(cfg: dict) -> dict:

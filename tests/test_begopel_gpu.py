@@ -130,7 +130,7 @@ def test_a_silenced_branch_and_a_cap_show_in_the_plain_model():
 
 # ------------------------------------------------------------------------------ prompts, decoding, portions
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("which", ["P", "Q", "R"])
+@pytest.mark.parametrize("which", ["P", "Q", "R", "S"])
 def test_prompt_decoding_and_portions(which, dtype):
     cfg, w, model = model_of(which, dtype)
     tokens = tokens_for(cfg, 150, 1)
