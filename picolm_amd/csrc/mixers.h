@@ -119,6 +119,136 @@ typedef struct {
 } picolm_map_rows_args;
 int picolm_call_map_rows(void* user, const picolm_step_view* v);
 
+
+// ---- row-wise steps of layers that norm after the sum, shift tokens and gate their branches ------
+
+// x[t][c] += sin(p f_i) for c = 2 i, cos(p f_i) for c = 2 i + 1, p the token's position.
+//   out: x float rows [width]
+typedef struct {
+    const double* freq;      // [ceil(width / 2)], f_i = base^(-2 i / width)
+    int32_t width;
+} picolm_add_positions_args;
+int picolm_call_add_positions(void* user, const picolm_step_view* v);
+
+// What a mixer reads where every token is blended with the one before it:
+//   y[t] = x[t] + (x[t-1] - x[t]) * mu, x[-1] of a sequence being what its state holds (zeros at the
+//   start); the state then takes the sequence's last x.
+//   in: x float rows [width]; out: y rows [width] in the engine's dtype; extra[0] (optional): x
+//   itself in the engine's dtype; state: floats [width] at state_off of the slot's state.
+typedef struct {
+    const float* mu;         // [width]
+    int32_t width;
+    int64_t state_off;       // in floats
+} picolm_token_shift_args;
+int picolm_call_token_shift(void* user, const picolm_step_view* v);
+
+// out[c] = x[c] * act(g[c] + bias[c]) over `width` columns; act 0: no gate (a copy into another
+// dtype or stride), 1: silu, 2: sigmoid.
+//   in: x rows [x_stride] of x_dtype, columns at x_off; extra[0]: g float rows [g_stride], columns at
+//   g_off (act > 0); out: rows [width] of out_dtype.
+typedef struct {
+    int32_t width, act;
+    int32_t x_stride, x_off, x_dtype;
+    int32_t g_stride, g_off;
+    int32_t out_dtype;
+    const float* bias;       // [width] or null
+} picolm_gate_rows_args;
+int picolm_call_gate_rows(void* user, const picolm_step_view* v);
+
+// RMS norm of a stretch of columns: out[out_off + c] = x[in_off + c] / sqrt(mean_c(x^2) + eps) * weight[c].
+//   in: float rows [in_stride]; out: rows [out_stride] of out_dtype.
+typedef struct {
+    const float* weight;     // [width]
+    int32_t width;
+    int32_t in_stride, in_off, out_stride, out_off, out_dtype;
+    float eps;
+} picolm_slice_norm_args;
+int picolm_call_slice_norm(void* user, const picolm_step_view* v);
+
+// A product per head: out[h] = W_h in[h] (transposed = 0: W [heads out_dim][in_dim]) or
+// out[h] = W_h^T in[h] (transposed = 1: W [heads in_dim][out_dim]), float accumulation, and then
+// out *= act(g) with g at the output's columns (gate_act 0: none, 1 silu, 2 sigmoid).
+//   in: rows [in_stride] of in_dtype, heads side by side at in_off; out: rows [out_stride] of
+//   out_dtype, heads side by side at out_off; extra[0]: g float rows [gate_stride], at gate_off.
+typedef struct {
+    const void* weight;
+    int32_t weight_dt;       // PICOLM_F32 / PICOLM_BF16
+    int32_t heads, in_dim, out_dim, transposed;
+    int32_t in_stride, in_off, in_dtype;
+    int32_t out_stride, out_off, out_dtype;
+    int32_t gate_act, gate_stride, gate_off;
+} picolm_head_linear_args;
+int picolm_call_head_linear(void* user, const picolm_step_view* v);
+
+// The sum and the norm of a layer that norms after adding:
+//   x <- (alpha x + u act(g + bias)) / rms(.) * weight          act = sigmoid where g is given, 1 else
+//   out: x float rows [width]; in: u float rows [width]; extra[0] (optional): g float rows [width].
+typedef struct {
+    const float* weight;     // [width]
+    const float* gate_bias;  // [width] or null
+    int32_t width;
+    float alpha, eps;
+} picolm_gated_postnorm_args;
+int picolm_call_gated_postnorm(void* user, const picolm_step_view* v);
+
+// What a matrix state with a forget gate per key channel needs of a token, from pre-activations:
+//   q = silu(q_raw);  a = lower + (1 - lower) sigmoid(f_raw + bias);  k = 1 - a
+//   in: float rows [in_stride], q_raw and f_raw [channels] at q_off, f_off; out: float rows
+//   [3 channels]: q | k | a.
+typedef struct {
+    const float* lower;      // [channels]
+    const float* bias;       // [channels] or null
+    int32_t channels, in_stride, q_off, f_off;
+} picolm_forget_gates_args;
+int picolm_call_forget_gates(void* user, const picolm_step_view* v);
+
+// A matrix state S [key_dim][value_dim] per head and sequence whose every element decays by a
+// factor of its own, walked over the step's tokens in order, kept in float in the slot's state:
+//   S[i][j] <- a[i][j] S[i][j] + k[i] w[j];   o[j] = sum_i S[i][j] q[i] + skip[j] x[j]
+//   kind 1: a[i][j] = a[i], a row's decay, given per token and key head; w = x
+//   kind 2: a[i][j] = exp(dt[j] A[j][i]), dt = softplus(dt_raw + dt_bias) per value channel; w = dt x
+//   extra[0]: float rows [qk_stride] with q, k (and kind 1: a) [key_heads][key_dim] at q_off, k_off,
+//   a_off; in: float rows [x_stride] with x [heads value_dim] at x_off; extra[1] (kind 2): float
+//   rows [dt_stride] with dt_raw [heads value_dim] at dt_off; out: float rows [heads value_dim].
+//   Head h uses q/k head h / (heads / key_heads).
+typedef struct {
+    int32_t kind;
+    int32_t n_heads, n_key_heads, key_dim, value_dim;
+    int32_t qk_stride, q_off, k_off, a_off;
+    int32_t x_stride, x_off;
+    int32_t dt_stride, dt_off;
+    const float* dt_bias;    // [heads value_dim] or null
+    const float* A;          // kind 2: [heads value_dim][key_dim], negative
+    const float* skip;       // [heads value_dim] or null
+    int64_t state_off;       // in floats: [heads][key_dim][value_dim]
+} picolm_decay_scan_args;
+int picolm_call_decay_scan(void* user, const picolm_step_view* v);
+
+// ---- a routed feed-forward ---------------------------------------------------------------------
+// Each row picks the `top` experts with the largest logits (ties: the lower index), weighted by
+// the softmax over the picked logits.
+//   in: float rows [experts] of router logits without bias; out: rows of 2 top words: the picked
+//   experts (int32) and then their weights (float).
+typedef struct {
+    const float* bias;       // [experts] or null
+    int32_t experts, top;
+} picolm_route_top_args;
+int picolm_call_route_top(void* user, const picolm_step_view* v);
+
+// The picked experts of every row: y[t][k] = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)), e the k-th
+// pick of row t, and their weighted sum  out[t] = sum_k w[t][k] y[t][k] (+ out[t] if `adds`).
+//   in: h rows [width] in the engine's dtype; extra[0]: the picks as route_top leaves them; extra[1]:
+//   scratch float rows [top width]; out: float rows [width].
+typedef struct {
+    const void* gate;        // [experts][ff][width]
+    const void* up;          // [experts][ff][width]
+    const void* down;        // [experts][width][ff]
+    int32_t weight_dt;
+    int32_t experts, top, width, ff;
+    int32_t adds;            // 1: out += the sum; 0: out = the sum
+} picolm_routed_experts_args;
+int picolm_call_routed_experts(void* user, const picolm_step_view* v);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,175 @@
+// A routed feed-forward (mixers.h): every row picks a few experts by its router logits and only
+// their weights are read.  Three kernels: the pick; the picked experts' hidden units (a workgroup
+// per (row, pick, 16 hidden units)); the down products with the weighted sum over a row's picks (a
+// workgroup per (row, 16 outputs)), so that a row's result is added up in one place and in a fixed
+// order.  A wave takes one weight row at a time, 16 bytes a lane, against the row's input in LDS.
+// Logits, picks, weights, hidden units and sums are float.
+#include "mixers.h"
+
+#include "api.h"
+#include "common.h"
+
+#define VIEW_REQUIRE(who, v)                                                                                      \
+    PICOLM_REQUIRE((v) && (v)->struct_bytes == (int32_t)sizeof(picolm_step_view), "%s: the step view is of another version", who)
+
+static inline int elem_bytes(int dt) { return dt == PICOLM_F32 ? 4 : 2; }
+
+// ---- the pick --------------------------------------------------------------------------------------
+// a thread a row; the picks come out in the order (logit falling, index rising)
+__global__ void route_top_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int32_t* __restrict__ out, int E, int top,
+                                 int n_rows) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n_rows) return;
+    const float* z = logits + (size_t)row * E;
+    int32_t* ids = out + (size_t)row * 2 * top;
+    float* w = (float*)(ids + top);
+    float last_z = INFINITY, first_z = 0.f, sum = 0.f;
+    int last_e = -1;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int be = -1;
+        for (int e = 0; e < E; ++e) {
+            const float ze = z[e] + (bias ? bias[e] : 0.f);
+            const bool after_last = ze < last_z || (ze == last_z && e > last_e);
+            if (after_last && (be < 0 || ze > best)) best = ze, be = e;
+        }
+        if (be < 0) be = k % E, best = -INFINITY;     // (only logits that are no numbers lead here)
+        if (k == 0) first_z = best;
+        const float p = expf(best - first_z);
+        ids[k] = be;
+        w[k] = p;
+        sum += p;
+        last_z = best, last_e = be;
+    }
+    for (int k = 0; k < top; ++k) w[k] /= sum;
+}
+
+extern "C" int picolm_call_route_top(void* user, const picolm_step_view* v) {
+    const picolm_route_top_args* a = (const picolm_route_top_args*)user;
+    VIEW_REQUIRE("route_top", v);
+    PICOLM_REQUIRE(a && v->in && v->out && a->experts > 0 && a->top > 0 && a->top <= a->experts, "route_top: %d picks among %d experts",
+                   a ? a->top : 0, a ? a->experts : 0);
+    PICOLM_REQUIRE(v->in_row_bytes >= a->experts * 4 && v->out_row_bytes >= 2 * a->top * 4, "route_top: rows too short");
+    if (v->rows <= 0) return 0;
+    route_top_kernel<<<ceil_div(v->rows, 64), 64, 0, v->stream>>>((const float*)v->in, a->bias, (int32_t*)v->out, a->experts, a->top, v->rows);
+    PICOLM_LAUNCH_CHECK("route_top");
+    return 0;
+}
+
+// ---- the picked experts ------------------------------------------------------------------------------
+// a lane's share of the dot product of a weight row with floats in LDS
+template <typename TW> __device__ __forceinline__ float lane_dot(const TW* __restrict__ w, const float* __restrict__ h, int K, int lane);
+template <> __device__ __forceinline__ float lane_dot<bf16_t>(const bf16_t* __restrict__ w, const float* __restrict__ h, int K, int lane) {
+    float acc = 0.f;
+    if (K % 8 == 0) {
+        for (int i = lane * 8; i < K; i += WAVE * 8) {
+            const uint4 p = *(const uint4*)(w + i);
+            const uint32_t u[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc += __uint_as_float(u[j] << 16) * h[i + 2 * j];
+                acc += __uint_as_float(u[j] & 0xffff0000u) * h[i + 2 * j + 1];
+            }
+        }
+    } else {
+        for (int i = lane; i < K; i += WAVE) acc += bf16_bits_to_f32(w[i]) * h[i];
+    }
+    return acc;
+}
+template <> __device__ __forceinline__ float lane_dot<float>(const float* __restrict__ w, const float* __restrict__ h, int K, int lane) {
+    float acc = 0.f;
+    if (K % 4 == 0) {
+        for (int i = lane * 4; i < K; i += WAVE * 4) {
+            const float4 p = *(const float4*)(w + i);
+            acc += p.x * h[i] + p.y * h[i + 1] + p.z * h[i + 2] + p.w * h[i + 3];
+        }
+    } else {
+        for (int i = lane; i < K; i += WAVE) acc += w[i] * h[i];
+    }
+    return acc;
+}
+
+#define MOE_UNITS 16     // hidden units, or outputs, a workgroup of four waves takes
+
+// act[row][pick][f] = silu(W_gate[e][f] . h) * (W_up[e][f] . h)
+template <typename TW, typename TH>
+__global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict__ h, const int32_t* __restrict__ picks, float* __restrict__ act,
+                                                            const TW* __restrict__ gate, const TW* __restrict__ up, int E, int top, int D, int F) {
+    extern __shared__ float moe_lds[];       // [D]
+    const int pair = blockIdx.x, row = pair / top, k = pair % top;
+    const int e = picks[(size_t)row * 2 * top + k];
+    for (int c = threadIdx.x; c < D; c += blockDim.x) moe_lds[c] = to_f32<TH>(h[(size_t)row * D + c]);
+    __syncthreads();
+    if (e < 0 || e >= E) return;
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int f1 = min(F, (int)(blockIdx.y + 1) * MOE_UNITS);
+    for (int f = blockIdx.y * MOE_UNITS + wave; f < f1; f += blockDim.x / WAVE) {
+        const size_t w_row = ((size_t)e * F + f) * D;
+        const float g = wave_sum(lane_dot<TW>(gate + w_row, moe_lds, D, lane));
+        const float u = wave_sum(lane_dot<TW>(up + w_row, moe_lds, D, lane));
+        if (lane == 0) act[((size_t)row * top + k) * F + f] = g / (1.f + expf(-g)) * u;
+    }
+}
+
+// out[row][d] (+)= sum_k w[row][k] (W_down[e_k][d] . act[row][k])
+template <typename TW>
+__global__ __launch_bounds__(256) void expert_down_kernel(const float* __restrict__ act, const int32_t* __restrict__ picks, float* __restrict__ out,
+                                                          const TW* __restrict__ down, int E, int top, int D, int F, int adds) {
+    extern __shared__ float moe_lds[];       // [top][F]
+    const int row = blockIdx.x;
+    for (int c = threadIdx.x; c < top * F; c += blockDim.x) moe_lds[c] = act[(size_t)row * top * F + c];
+    __syncthreads();
+    const int32_t* ids = picks + (size_t)row * 2 * top;
+    const float* w = (const float*)(ids + top);
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int d1 = min(D, (int)(blockIdx.y + 1) * MOE_UNITS);
+    for (int d = blockIdx.y * MOE_UNITS + wave; d < d1; d += blockDim.x / WAVE) {
+        float total = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = ids[k];
+            if (e < 0 || e >= E) continue;
+            total += w[k] * wave_sum(lane_dot<TW>(down + ((size_t)e * D + d) * F, moe_lds + (size_t)k * F, F, lane));
+        }
+        if (lane == 0) out[(size_t)row * D + d] = (adds ? out[(size_t)row * D + d] : 0.f) + total;
+    }
+}
+
+extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v) {
+    const picolm_routed_experts_args* a = (const picolm_routed_experts_args*)user;
+    VIEW_REQUIRE("routed_experts", v);
+    PICOLM_REQUIRE(a && a->gate && a->up && a->down && v->in && v->out && v->extra[0] && v->extra[1], "routed_experts: weights or buffers are missing");
+    const int E = a->experts, top = a->top, D = a->width, F = a->ff;
+    PICOLM_REQUIRE(E > 0 && top > 0 && top <= E && D > 0 && F > 0 && (a->weight_dt == PICOLM_F32 || a->weight_dt == PICOLM_BF16),
+                   "routed_experts: %d picks among %d experts of %d to %d", top, E, D, F);
+    PICOLM_REQUIRE(v->dtype == PICOLM_BF16 || a->weight_dt == PICOLM_F32, "routed_experts: the 32-bit engine takes 32-bit weights");
+    PICOLM_REQUIRE(v->in_row_bytes >= D * elem_bytes(v->dtype) && v->out_row_bytes >= D * 4 && v->extra_row_bytes[0] >= 2 * top * 4 &&
+                       v->extra_row_bytes[1] >= (int64_t)top * F * 4,
+                   "routed_experts: rows too short for a width of %d, %d picks and %d hidden units", D, top, F);
+    const size_t lds_a = sizeof(float) * (size_t)D, lds_b = sizeof(float) * (size_t)top * F;
+    PICOLM_REQUIRE(lds_a <= 64 * 1024 && lds_b <= 64 * 1024, "routed_experts: a width of %d or %d picks of %d hidden units exceed 64 KiB of LDS", D,
+                   top, F);
+    PICOLM_REQUIRE(ceil_div(F, MOE_UNITS) <= 65535 && ceil_div(D, MOE_UNITS) <= 65535 && (int64_t)v->rows * top < (1ll << 31),
+                   "routed_experts: the sizes exceed the grid");
+    if (v->rows <= 0) return 0;
+    const int32_t* picks = (const int32_t*)v->extra[0];
+    float* act = (float*)v->extra[1];
+    const dim3 grid_a((unsigned)(v->rows * top), ceil_div(F, MOE_UNITS)), grid_b(v->rows, ceil_div(D, MOE_UNITS));
+    if (a->weight_dt == PICOLM_F32 && v->dtype == PICOLM_F32) {
+        expert_hidden_kernel<float, float><<<grid_a, 256, lds_a, v->stream>>>((const float*)v->in, picks, act, (const float*)a->gate,
+                                                                              (const float*)a->up, E, top, D, F);
+        PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
+        expert_down_kernel<float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds);
+    } else if (a->weight_dt == PICOLM_F32) {
+        expert_hidden_kernel<float, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const float*)a->gate,
+                                                                               (const float*)a->up, E, top, D, F);
+        PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
+        expert_down_kernel<float><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const float*)a->down, E, top, D, F, a->adds);
+    } else {
+        expert_hidden_kernel<bf16_t, bf16_t><<<grid_a, 256, lds_a, v->stream>>>((const bf16_t*)v->in, picks, act, (const bf16_t*)a->gate,
+                                                                                (const bf16_t*)a->up, E, top, D, F);
+        PICOLM_LAUNCH_CHECK("routed_experts (hidden)");
+        expert_down_kernel<bf16_t><<<grid_b, 256, lds_b, v->stream>>>(act, picks, (float*)v->out, (const bf16_t*)a->down, E, top, D, F, a->adds);
+    }
+    PICOLM_LAUNCH_CHECK("routed_experts (down)");
+    return 0;
+}

@@ -1,0 +1,325 @@
+// Called operations of the library's own (mixers.h) that work row by row: positions added to the
+// embedding, the blend of a token with the one before it, gates, norms of a stretch of columns, a
+// product per head, and the sum-then-norm of layers that norm after adding.  Every function checks
+// what it is handed on the host, then queues its kernels on the step's stream; what they do
+// depends on device memory only, so a decode step that holds them can be recorded and replayed.
+//
+// All arithmetic is float (angles double); rows that feed a product are written in the engine's dtype.
+#include "mixers.h"
+
+#include "api.h"
+#include "common.h"
+
+#define VIEW_REQUIRE(who, v)                                                                                      \
+    PICOLM_REQUIRE((v) && (v)->struct_bytes == (int32_t)sizeof(picolm_step_view), "%s: the step view is of another version", who)
+
+static inline int elem_bytes(int dt) { return dt == PICOLM_F32 ? 4 : 2; }
+static inline bool known_dtype(int dt) { return dt == PICOLM_F32 || dt == PICOLM_BF16; }
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
+
+// an element of a buffer whose dtype is known at run time
+__device__ __forceinline__ float load_as_f32(const void* p, size_t i, int dt) {
+    return dt == PICOLM_F32 ? ((const float*)p)[i] : bf16_bits_to_f32(((const bf16_t*)p)[i]);
+}
+__device__ __forceinline__ void store_from_f32(void* p, size_t i, int dt, float v) {
+    if (dt == PICOLM_F32) ((float*)p)[i] = v;
+    else ((bf16_t*)p)[i] = f32_to_bf16_bits(v);
+}
+
+// ---- positions ------------------------------------------------------------------------------------
+__global__ void add_positions_kernel(float* __restrict__ x, const int32_t* __restrict__ tok_pos, const double* __restrict__ freq, int W) {
+    const size_t row = blockIdx.x;
+    const double p = (double)tok_pos[row];
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const double angle = p * freq[c >> 1];
+        x[row * W + c] += (float)((c & 1) ? cos(angle) : sin(angle));
+    }
+}
+
+extern "C" int picolm_call_add_positions(void* user, const picolm_step_view* v) {
+    const picolm_add_positions_args* a = (const picolm_add_positions_args*)user;
+    VIEW_REQUIRE("add_positions", v);
+    PICOLM_REQUIRE(a && a->freq && a->width > 0 && v->out && v->tok_pos, "add_positions: the table or the rows are missing");
+    PICOLM_REQUIRE(v->out_row_bytes >= a->width * 4, "add_positions: rows too short for a width of %d", a->width);
+    if (v->rows <= 0) return 0;
+    add_positions_kernel<<<v->rows, 256, 0, v->stream>>>((float*)v->out, v->tok_pos, a->freq, a->width);
+    PICOLM_LAUNCH_CHECK("add_positions");
+    return 0;
+}
+
+// ---- a token blended with the one before it ---------------------------------------------------------
+// One workgroup a row.  A sequence that brings one token reads its state and then writes it in the
+// same thread; the state of a sequence that brings more is written by the kernel after this one.
+template <typename T>
+__global__ void token_shift_kernel(const float* __restrict__ x, T* __restrict__ y, T* __restrict__ plain, float* __restrict__ state,
+                                   int64_t slot_floats, const float* __restrict__ mu, int W, const int32_t* __restrict__ tok_seq,
+                                   const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot) {
+    const int row = blockIdx.x;
+    const int seq = tok_seq[row], first = cu_seqlens[seq], n = cu_seqlens[seq + 1] - first;
+    float* st = state + (size_t)seq_slot[seq] * slot_floats;
+    const float* prev = row > first ? x + (size_t)(row - 1) * W : st;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float xv = x[(size_t)row * W + c], pv = prev[c];
+        y[(size_t)row * W + c] = from_f32<T>(xv + (pv - xv) * mu[c]);
+        if (plain) plain[(size_t)row * W + c] = from_f32<T>(xv);
+        if (n == 1) st[c] = xv;
+    }
+}
+
+__global__ void token_shift_state_kernel(const float* __restrict__ x, float* __restrict__ state, int64_t slot_floats, int W,
+                                         const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_slot) {
+    const int seq = blockIdx.x;
+    const int first = cu_seqlens[seq], n = cu_seqlens[seq + 1] - first;
+    if (n <= 1) return;
+    float* st = state + (size_t)seq_slot[seq] * slot_floats;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) st[c] = x[(size_t)(first + n - 1) * W + c];
+}
+
+extern "C" int picolm_call_token_shift(void* user, const picolm_step_view* v) {
+    const picolm_token_shift_args* a = (const picolm_token_shift_args*)user;
+    VIEW_REQUIRE("token_shift", v);
+    PICOLM_REQUIRE(a && a->mu && a->width > 0 && v->in && v->out && v->state, "token_shift: weights, buffers or state are missing");
+    const int es = elem_bytes(v->dtype), W = a->width;
+    PICOLM_REQUIRE(v->in_row_bytes >= W * 4 && v->out_row_bytes >= W * es && (!v->extra[0] || v->extra_row_bytes[0] >= W * es),
+                   "token_shift: rows too short for a width of %d", W);
+    PICOLM_REQUIRE(a->state_off >= 0 && (a->state_off + W) * 4 <= v->state_bytes_per_slot,
+                   "token_shift: the state of a slot has %lld bytes, a row at %lld needs %lld", (long long)v->state_bytes_per_slot,
+                   (long long)a->state_off, (long long)((a->state_off + W) * 4));
+    if (v->n_tokens <= 0) return 0;
+    const int64_t slot_floats = v->state_bytes_per_slot / 4;
+    float* state = (float*)v->state + a->state_off;
+    if (v->dtype == PICOLM_F32)
+        token_shift_kernel<float><<<v->n_tokens, 256, 0, v->stream>>>((const float*)v->in, (float*)v->out, (float*)v->extra[0], state, slot_floats,
+                                                                     a->mu, W, v->tok_seq, v->cu_seqlens, v->seq_slot);
+    else
+        token_shift_kernel<bf16_t><<<v->n_tokens, 256, 0, v->stream>>>((const float*)v->in, (bf16_t*)v->out, (bf16_t*)v->extra[0], state,
+                                                                      slot_floats, a->mu, W, v->tok_seq, v->cu_seqlens, v->seq_slot);
+    PICOLM_LAUNCH_CHECK("token_shift");
+    if (!v->is_decode) {
+        token_shift_state_kernel<<<v->n_seq, 256, 0, v->stream>>>((const float*)v->in, state, slot_floats, W, v->cu_seqlens, v->seq_slot);
+        PICOLM_LAUNCH_CHECK("token_shift (state)");
+    }
+    return 0;
+}
+
+// ---- a gate over columns ---------------------------------------------------------------------------
+__global__ void gate_rows_kernel(const void* __restrict__ x, int x_stride, int x_off, int x_dt, const float* __restrict__ g, int g_stride,
+                                 int g_off, const float* __restrict__ bias, void* __restrict__ out, int out_dt, int W, int act, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const size_t row = i / W;
+        const int c = (int)(i % W);
+        float y = load_as_f32(x, row * x_stride + x_off + c, x_dt);
+        if (act) {
+            const float z = g[row * g_stride + g_off + c] + (bias ? bias[c] : 0.f);
+            y *= act == 1 ? silu_f(z) : sigmoid_f(z);
+        }
+        store_from_f32(out, (size_t)i, out_dt, y);
+    }
+}
+
+extern "C" int picolm_call_gate_rows(void* user, const picolm_step_view* v) {
+    const picolm_gate_rows_args* a = (const picolm_gate_rows_args*)user;
+    VIEW_REQUIRE("gate_rows", v);
+    PICOLM_REQUIRE(a && v->in && v->out && a->width > 0 && a->act >= 0 && a->act <= 2 && known_dtype(a->x_dtype) && known_dtype(a->out_dtype),
+                   "gate_rows: buffers are missing, or an unknown gate or dtype");
+    PICOLM_REQUIRE(a->x_off >= 0 && a->x_off + a->width <= a->x_stride && v->in_row_bytes >= a->x_stride * elem_bytes(a->x_dtype) &&
+                       v->out_row_bytes >= a->width * elem_bytes(a->out_dtype),
+                   "gate_rows: rows too short for %d columns at %d of %d", a->width, a->x_off, a->x_stride);
+    PICOLM_REQUIRE(!a->act || (v->extra[0] && a->g_off >= 0 && a->g_off + a->width <= a->g_stride && v->extra_row_bytes[0] >= a->g_stride * 4),
+                   "gate_rows: the gate's rows of %d floats do not hold %d at %d", a->g_stride, a->width, a->g_off);
+    if (v->rows <= 0) return 0;
+    const int64_t n = (int64_t)v->rows * a->width;
+    const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(n, 256), 65536);
+    gate_rows_kernel<<<blocks, 256, 0, v->stream>>>(v->in, a->x_stride, a->x_off, a->x_dtype, (const float*)v->extra[0], a->g_stride, a->g_off,
+                                                   a->bias, v->out, a->out_dtype, a->width, a->act, n);
+    PICOLM_LAUNCH_CHECK("gate_rows");
+    return 0;
+}
+
+// ---- the norm of a stretch of columns ------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void slice_norm_kernel(const float* __restrict__ x, int in_stride, int in_off, void* __restrict__ out,
+                                                         int out_stride, int out_off, int out_dt, const float* __restrict__ weight, int W,
+                                                         float eps) {
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    const float* xr = x + row * in_stride + in_off;
+    float ssq = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) ssq += xr[c] * xr[c];
+    ssq = block_sum(ssq, scratch);
+    const float inv = 1.f / sqrtf(ssq / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += blockDim.x) store_from_f32(out, row * out_stride + out_off + c, out_dt, xr[c] * inv * weight[c]);
+}
+
+extern "C" int picolm_call_slice_norm(void* user, const picolm_step_view* v) {
+    const picolm_slice_norm_args* a = (const picolm_slice_norm_args*)user;
+    VIEW_REQUIRE("slice_norm", v);
+    PICOLM_REQUIRE(a && a->weight && v->in && v->out && a->width > 0 && known_dtype(a->out_dtype), "slice_norm: weights or buffers are missing");
+    PICOLM_REQUIRE(a->in_off >= 0 && a->in_off + a->width <= a->in_stride && v->in_row_bytes >= a->in_stride * 4 && a->out_off >= 0 &&
+                       a->out_off + a->width <= a->out_stride && v->out_row_bytes >= a->out_stride * elem_bytes(a->out_dtype),
+                   "slice_norm: rows too short for %d columns at the offsets named", a->width);
+    PICOLM_REQUIRE(v->in != v->out, "slice_norm: input and output differ");
+    if (v->rows <= 0) return 0;
+    slice_norm_kernel<<<v->rows, a->width >= 2048 ? 1024 : 256, 0, v->stream>>>((const float*)v->in, a->in_stride, a->in_off, v->out, a->out_stride,
+                                                                               a->out_off, a->out_dtype, a->weight, a->width, a->eps);
+    PICOLM_LAUNCH_CHECK("slice_norm");
+    return 0;
+}
+
+// ---- a product per head -----------------------------------------------------------------------------
+// One workgroup per (HL_ROWS rows, head): the rows' inputs wait in LDS as floats and every weight
+// that is read meets all of them.  Not transposed: a wave per output, its lanes along the input;
+// transposed: a thread per output, adjacent threads read adjacent weights.
+#define HL_ROWS 8
+template <typename TW>
+__global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_args a, const void* __restrict__ in, void* __restrict__ out,
+                                                          const float* __restrict__ gate, int n_rows) {
+    extern __shared__ float hl_in[];      // [HL_ROWS][in_dim]
+    const int head = blockIdx.y, row0 = blockIdx.x * HL_ROWS, nr = min(HL_ROWS, n_rows - row0);
+    const int K = a.in_dim, N = a.out_dim;
+    for (int idx = threadIdx.x; idx < HL_ROWS * K; idx += blockDim.x) {
+        const int r = idx / K, i = idx % K;
+        hl_in[idx] = r < nr ? load_as_f32(in, (size_t)(row0 + r) * a.in_stride + a.in_off + (size_t)head * K + i, a.in_dtype) : 0.f;
+    }
+    __syncthreads();
+    const TW* w = (const TW*)a.weight;
+    auto finish = [&](int r, int o, float acc) {
+        const size_t row = row0 + r;
+        if (a.gate_act) {
+            const float z = gate[row * a.gate_stride + a.gate_off + (size_t)head * N + o];
+            acc *= a.gate_act == 1 ? silu_f(z) : sigmoid_f(z);
+        }
+        store_from_f32(out, row * a.out_stride + a.out_off + (size_t)head * N + o, a.out_dtype, acc);
+    };
+    if (a.transposed) {
+        const TW* wh = w + (size_t)head * K * N;
+        for (int o = threadIdx.x; o < N; o += blockDim.x) {
+            float acc[HL_ROWS];
+#pragma unroll
+            for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
+            for (int i = 0; i < K; ++i) {
+                const float wv = to_f32<TW>(wh[(size_t)i * N + o]);
+#pragma unroll
+                for (int r = 0; r < HL_ROWS; ++r) acc[r] += wv * hl_in[r * K + i];
+            }
+#pragma unroll
+            for (int r = 0; r < HL_ROWS; ++r)
+                if (r < nr) finish(r, o, acc[r]);
+        }
+    } else {
+        const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n_waves = blockDim.x / WAVE;
+        const TW* wh = w + (size_t)head * N * K;
+        for (int o = wave; o < N; o += n_waves) {
+            float acc[HL_ROWS];
+#pragma unroll
+            for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
+            for (int i = lane; i < K; i += WAVE) {
+                const float wv = to_f32<TW>(wh[(size_t)o * K + i]);
+#pragma unroll
+                for (int r = 0; r < HL_ROWS; ++r) acc[r] += wv * hl_in[r * K + i];
+            }
+#pragma unroll
+            for (int r = 0; r < HL_ROWS; ++r) {
+                const float s = wave_sum(acc[r]);
+                if (lane == 0 && r < nr) finish(r, o, s);
+            }
+        }
+    }
+}
+
+extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
+    const picolm_head_linear_args* a = (const picolm_head_linear_args*)user;
+    VIEW_REQUIRE("head_linear", v);
+    PICOLM_REQUIRE(a && a->weight && v->in && v->out && v->in != v->out, "head_linear: weights or buffers are missing (input and output differ)");
+    PICOLM_REQUIRE(a->heads > 0 && a->heads <= 65535 && a->in_dim > 0 && a->out_dim > 0 && known_dtype(a->weight_dt) && known_dtype(a->in_dtype) &&
+                       known_dtype(a->out_dtype) && a->gate_act >= 0 && a->gate_act <= 2,
+                   "head_linear: %d heads of %d to %d, or an unknown dtype or gate", a->heads, a->in_dim, a->out_dim);
+    PICOLM_REQUIRE(a->in_off >= 0 && a->in_off + (int64_t)a->heads * a->in_dim <= a->in_stride &&
+                       v->in_row_bytes >= (int64_t)a->in_stride * elem_bytes(a->in_dtype) && a->out_off >= 0 &&
+                       a->out_off + (int64_t)a->heads * a->out_dim <= a->out_stride &&
+                       v->out_row_bytes >= (int64_t)a->out_stride * elem_bytes(a->out_dtype),
+                   "head_linear: rows too short for %d heads at the offsets named", a->heads);
+    PICOLM_REQUIRE(!a->gate_act || (v->extra[0] && a->gate_off >= 0 && a->gate_off + (int64_t)a->heads * a->out_dim <= a->gate_stride &&
+                                    v->extra_row_bytes[0] >= (int64_t)a->gate_stride * 4),
+                   "head_linear: the gate's rows of %d floats do not hold the heads at %d", a->gate_stride, a->gate_off);
+    const size_t lds = sizeof(float) * HL_ROWS * (size_t)a->in_dim;
+    PICOLM_REQUIRE(lds <= 64 * 1024, "head_linear: an input of %d a head needs %zu bytes of LDS", a->in_dim, lds);
+    if (v->rows <= 0) return 0;
+    const dim3 grid(ceil_div(v->rows, HL_ROWS), a->heads);
+    if (a->weight_dt == PICOLM_F32)
+        head_linear_kernel<float><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);
+    else
+        head_linear_kernel<bf16_t><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);
+    PICOLM_LAUNCH_CHECK("head_linear");
+    return 0;
+}
+
+// ---- the sum and the norm of a layer that norms after adding ---------------------------------------------
+__global__ __launch_bounds__(1024) void gated_postnorm_kernel(float* __restrict__ x, const float* __restrict__ u, const float* __restrict__ g,
+                                                             const float* __restrict__ bias, const float* __restrict__ weight, int W,
+                                                             float alpha, float eps) {
+    __shared__ float scratch[16];
+    const size_t row = blockIdx.x;
+    float* xr = x + row * W;
+    const float* ur = u + row * W;
+    const float* gr = g ? g + row * W : nullptr;
+    auto sum_at = [&](int c) {
+        float uv = ur[c];
+        if (gr) uv *= sigmoid_f(gr[c] + (bias ? bias[c] : 0.f));
+        return alpha * xr[c] + uv;
+    };
+    float ssq = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float s = sum_at(c);
+        ssq += s * s;
+    }
+    ssq = block_sum(ssq, scratch);
+    const float inv = 1.f / sqrtf(ssq / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += blockDim.x) xr[c] = sum_at(c) * inv * weight[c];      // a thread writes what only it reads
+}
+
+extern "C" int picolm_call_gated_postnorm(void* user, const picolm_step_view* v) {
+    const picolm_gated_postnorm_args* a = (const picolm_gated_postnorm_args*)user;
+    VIEW_REQUIRE("gated_postnorm", v);
+    PICOLM_REQUIRE(a && a->weight && v->in && v->out && a->width > 0, "gated_postnorm: weights or buffers are missing");
+    PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * 4 && (!v->extra[0] || v->extra_row_bytes[0] >= a->width * 4),
+                   "gated_postnorm: rows too short for a width of %d", a->width);
+    if (v->rows <= 0) return 0;
+    gated_postnorm_kernel<<<v->rows, a->width >= 2048 ? 1024 : 256, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0],
+                                                                                   a->gate_bias, a->weight, a->width, a->alpha, a->eps);
+    PICOLM_LAUNCH_CHECK("gated_postnorm");
+    return 0;
+}
+
+// ---- what a forget gate per key channel gives a token --------------------------------------------------
+__global__ void forget_gates_kernel(const float* __restrict__ in, int in_stride, int q_off, int f_off, float* __restrict__ out,
+                                    const float* __restrict__ lower, const float* __restrict__ bias, int C, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const size_t row = i / C;
+        const int c = (int)(i % C);
+        const float* r = in + row * in_stride;
+        const float lo = lower[c];
+        const float a = lo + (1.f - lo) * sigmoid_f(r[f_off + c] + (bias ? bias[c] : 0.f));
+        float* o = out + row * 3 * C;
+        o[c] = silu_f(r[q_off + c]);
+        o[C + c] = 1.f - a;
+        o[2 * C + c] = a;
+    }
+}
+
+extern "C" int picolm_call_forget_gates(void* user, const picolm_step_view* v) {
+    const picolm_forget_gates_args* a = (const picolm_forget_gates_args*)user;
+    VIEW_REQUIRE("forget_gates", v);
+    PICOLM_REQUIRE(a && a->lower && v->in && v->out && v->in != v->out && a->channels > 0, "forget_gates: bounds or buffers are missing");
+    PICOLM_REQUIRE(a->q_off >= 0 && a->q_off + a->channels <= a->in_stride && a->f_off >= 0 && a->f_off + a->channels <= a->in_stride &&
+                       v->in_row_bytes >= a->in_stride * 4 && v->out_row_bytes >= (int64_t)3 * a->channels * 4,
+                   "forget_gates: rows too short for %d channels at the offsets named", a->channels);
+    if (v->rows <= 0) return 0;
+    const int64_t n = (int64_t)v->rows * a->channels;
+    const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(n, 256), 65536);
+    forget_gates_kernel<<<blocks, 256, 0, v->stream>>>((const float*)v->in, a->in_stride, a->q_off, a->f_off, (float*)v->out, a->lower, a->bias,
+                                                      a->channels, n);
+    PICOLM_LAUNCH_CHECK("forget_gates");
+    return 0;
+}

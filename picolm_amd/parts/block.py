@@ -42,6 +42,118 @@ class PreNormBlock(Block):
         self.ffn.emit(b, self.ffn_norm.emit(b, x), x, after, after_when)
 
 
+class _WithRowState(Mixer):
+    """A mixer as the cache sees it when its block keeps `row_floats` floats of its own per
+    sequence in front of the mixer's state: one state entry holds both."""
+
+    def __init__(self, inner: Mixer, row_floats: int):
+        self.inner, self.row_floats = inner, int(row_floats)
+        if self.row_floats and hasattr(inner, "state_base"):
+            inner.state_base = self.row_floats
+
+    def cache_requests(self):
+        import torch
+        from .base import StateRequest
+        kv, st = self.inner.cache_requests()
+        if not self.row_floats:
+            return kv, st
+        if st is not None and (len(st.shape) != 1 or st.dtype != torch.float32 or not hasattr(self.inner, "state_base")):
+            raise ValueError(f"{type(self.inner).__name__} keeps a state that a row cannot be put in front of")
+        return kv, StateRequest((self.row_floats + (st.shape[0] if st is not None else 0),), torch.float32)
+
+    def prepare(self, runtime, max_positions: int) -> None:
+        self.inner.prepare(runtime, max_positions)
+
+
+class PostNormBlock(Block):
+    """Norm after the sum, each branch reading the residual rows themselves:
+        x <- norm1(alpha x + gate1(x) * mixer(shifted(x)));   x <- norm2(alpha x + gate2(x) * ffn(x))
+    shifted(x)[t] = x[t] + (x[t-1] - x[t]) * mu (`shift_name`: the tensor mu; None: the mixer reads x),
+    with the row before a step's first one kept in the layer call's state; gate(x) = sigmoid(W x + b)
+    (`gate_names`: the two matrices, their biases at `<name>.b`; None: no gates).  A block without a
+    feed-forward has the first half only."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, hidden_size: int, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None, ffn: FeedForward | None,
+                 alpha: float = 1.0, shift_name: str | None = None, gate_names=None):
+        from .linear import Linear
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.D, self.alpha = hidden_size, float(alpha)
+        self.mixer_norm, self.inner, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+        self.shift_name = shift_name
+        self.mixer = _WithRowState(mixer, hidden_size if shift_name else 0)
+        self.gate_names = tuple(gate_names) if gate_names else None
+        self.gates = [Linear([n], [hidden_size], hidden_size) for n in self.gate_names[:2 if ffn is not None else 1]] if gate_names else []
+        self.mu = None
+        self.gate_bias = []
+
+    def children(self):
+        return [p for p in (self.mixer_norm, self.inner, self.ffn_norm, self.ffn, *self.gates) if p is not None]
+
+    def tensor_specs(self):
+        from ..weights import TensorSpec
+        specs = [TensorSpec(self.shift_name, (self.D,))] if self.shift_name else []
+        specs += [TensorSpec(g.names[0] + ".b", (self.D,), init="zeros") for g in self.gates]
+        if self.gate_names and len(self.gates) < len(self.gate_names):      # a block without a feed-forward may carry its gate all the same
+            specs += [TensorSpec(n + s, shape, optional=True, init=None) for n in self.gate_names[len(self.gates):]
+                      for s, shape in (("", (self.D, self.D)), (".b", (self.D,)))]
+        return specs
+
+    def load(self, fetch, runtime) -> None:
+        import torch
+        if self.shift_name:
+            self.mu = fetch.get(self.shift_name).to(torch.float32).contiguous()
+        self.gate_bias = [fetch.get(g.names[0] + ".b").to(torch.float32).contiguous() for g in self.gates]
+
+    def _join(self, b, x: int, branch: int, plain: int, which: int, norm) -> None:
+        """x <- norm(alpha x + branch * gate(plain))"""
+        import torch
+        from .. import kernels
+        from .calls import GatedPostnormArgs, emit_library_call
+        extra, bias = [], None
+        if self.gates:
+            g = b.buffer("postnorm.gate", self.D, torch.float32)
+            self.gates[which].emit(b, plain, g, kernels.EPI_STORE)
+            extra, bias = [g], self.gate_bias[which]
+        ref = norm.norm_ref()
+        if ref is None:
+            raise ValueError("a block that norms after the sum takes RMS norms")
+        emit_library_call(b, "gated_postnorm", GatedPostnormArgs(b._ptr(ref.weight), b._ptr(bias), self.D, self.alpha, ref.eps), x,
+                          inp=branch, extra=extra)
+
+    def _plain_rows(self, b, x: int) -> int:
+        """The residual rows in the dtype that products read."""
+        import torch
+        from ..engine.program import _DT, F32
+        from .calls import GATE_NONE, GateRowsArgs, emit_library_call
+        plain = b.buffer("postnorm.plain", self.D, b.dtype)
+        emit_library_call(b, "gate_rows", GateRowsArgs(self.D, GATE_NONE, self.D, 0, F32, 0, 0, _DT[b.dtype], None), plain, inp=x)
+        return plain
+
+    def emit(self, b, x: int, after=None, after_when: int = 0) -> None:
+        import torch
+        from ..engine.program import Rows
+        from .calls import TokenShiftArgs, emit_library_call
+        D = self.D
+        if self.shift_name:
+            if self.mu is None:
+                raise ValueError(f"{self.shift_name} is not loaded")
+            plain = b.buffer("postnorm.plain", D, b.dtype)
+            reads = b.buffer("postnorm.shifted", D, b.dtype)
+            emit_library_call(b, "token_shift", TokenShiftArgs(b._ptr(self.mu), D, 0), reads, inp=x, extra=[plain] if self.gates else [],
+                              uses_state=True)
+        else:
+            plain = reads = self._plain_rows(b, x)
+        branch = b.buffer("postnorm.branch", D, torch.float32)
+        self.inner.emit(b, Rows(reads), branch, accumulate=False)
+        self._join(b, x, branch, plain, 0, self.mixer_norm)
+        if self.ffn is not None:
+            plain = self._plain_rows(b, x)
+            self.ffn.emit(b, Rows(plain), branch, accumulate=False)
+            self._join(b, x, branch, plain, 1, self.ffn_norm)
+
+
 class _NoMixer(Mixer):
     """The mixer of a block that has none: it asks nothing of the cache."""
 

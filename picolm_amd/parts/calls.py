@@ -46,6 +46,59 @@ class MapRowsArgs(Structure):
     _fields_ = [("kind", c_int32), ("width", c_int32), ("in_dtype", c_int32), ("out_dtype", c_int32), ("param", c_float)]
 
 
+class AddPositionsArgs(Structure):
+    _fields_ = [("freq", c_void_p), ("width", c_int32)]
+
+
+class TokenShiftArgs(Structure):
+    _fields_ = [("mu", c_void_p), ("width", c_int32), ("state_off", c_int64)]
+
+
+class GateRowsArgs(Structure):
+    _fields_ = [("width", c_int32), ("act", c_int32), ("x_stride", c_int32), ("x_off", c_int32), ("x_dtype", c_int32),
+                ("g_stride", c_int32), ("g_off", c_int32), ("out_dtype", c_int32), ("bias", c_void_p)]
+
+
+class SliceNormArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("width", c_int32), ("in_stride", c_int32), ("in_off", c_int32), ("out_stride", c_int32),
+                ("out_off", c_int32), ("out_dtype", c_int32), ("eps", c_float)]
+
+
+class HeadLinearArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("weight_dt", c_int32), ("heads", c_int32), ("in_dim", c_int32), ("out_dim", c_int32),
+                ("transposed", c_int32), ("in_stride", c_int32), ("in_off", c_int32), ("in_dtype", c_int32),
+                ("out_stride", c_int32), ("out_off", c_int32), ("out_dtype", c_int32),
+                ("gate_act", c_int32), ("gate_stride", c_int32), ("gate_off", c_int32)]
+
+
+class GatedPostnormArgs(Structure):
+    _fields_ = [("weight", c_void_p), ("gate_bias", c_void_p), ("width", c_int32), ("alpha", c_float), ("eps", c_float)]
+
+
+class ForgetGatesArgs(Structure):
+    _fields_ = [("lower", c_void_p), ("bias", c_void_p), ("channels", c_int32), ("in_stride", c_int32), ("q_off", c_int32),
+                ("f_off", c_int32)]
+
+
+class DecayScanArgs(Structure):
+    _fields_ = [("kind", c_int32), ("n_heads", c_int32), ("n_key_heads", c_int32), ("key_dim", c_int32), ("value_dim", c_int32),
+                ("qk_stride", c_int32), ("q_off", c_int32), ("k_off", c_int32), ("a_off", c_int32),
+                ("x_stride", c_int32), ("x_off", c_int32), ("dt_stride", c_int32), ("dt_off", c_int32),
+                ("dt_bias", c_void_p), ("A", c_void_p), ("skip", c_void_p), ("state_off", c_int64)]
+
+
+class RouteTopArgs(Structure):
+    _fields_ = [("bias", c_void_p), ("experts", c_int32), ("top", c_int32)]
+
+
+class RoutedExpertsArgs(Structure):
+    _fields_ = [("gate", c_void_p), ("up", c_void_p), ("down", c_void_p), ("weight_dt", c_int32), ("experts", c_int32),
+                ("top", c_int32), ("width", c_int32), ("ff", c_int32), ("adds", c_int32)]
+
+
+GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2
+DECAY_PER_ROW, DECAY_EXPONENTIAL = 1, 2
+DECAY_SCAN_MAX_KEY_DIM = 256
 MAP_RELU_SQUARED, MAP_SOFTCAP = 1, 2
 RULE_OUTER_PRODUCT, RULE_DELTA = 0, 1
 STATE_SCAN_MAX_KEY_DIM = 256

@@ -14,12 +14,18 @@ from .base import Part, Runtime
 class TokenEmbedding(Part):
     graph_safe = True      # launches depend on device memory only
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0, keeps_output: bool = False):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0, keeps_output: bool = False,
+                 positions: "SinusoidalPositions | None" = None):
         """`scale`: the rows are multiplied by it (in float).  `keeps_output`: the output is also
-        left in a buffer of its own (`embed.out`), for parts that read it again later."""
+        left in a buffer of its own (`embed.out`), for parts that read it again later.  `positions`:
+        a vector per position that is added to the rows."""
         self.name, self.V, self.D = name, vocab_size, hidden_size
         self.scale, self.keeps_output = float(scale), bool(keeps_output)
+        self.positions = positions
         self.table = None
+
+    def children(self):
+        return [self.positions] if self.positions is not None else []
 
     def tensor_specs(self):
         return [TensorSpec(self.name, (self.V, self.D))]
@@ -34,6 +40,8 @@ class TokenEmbedding(Part):
             raise ValueError(f"embedding {self.name} has no table loaded")
         x = b.buffer("residual", self.D, torch.float32)
         b.embed(self.table, x, self.scale)
+        if self.positions is not None:
+            self.positions.emit(b, x)
         if self.keeps_output:
             b.embed(self.table, b.buffer("embed.out", self.D, torch.float32), self.scale)
         return x
@@ -43,6 +51,28 @@ class TokenEmbedding(Part):
         kernels.embed(self.table, tokens, x)
         if self.scale != 1.0:
             x.mul_(self.scale)
+
+
+class SinusoidalPositions(Part):
+    """A fixed vector per position, added to the embedding: entry 2i is sin(p f_i), entry 2i+1 is
+    cos(p f_i) with f_i = base^(-2i / width).  The frequencies are laid out once, in double; the
+    angle of a token is taken in double from its position in the step's arrays, so the part has no
+    table that a longest sequence would size."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, width: int, base: float = 10000.0):
+        self.width, self.base = int(width), float(base)
+        self.freq = None
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        i = torch.arange((self.width + 1) // 2, dtype=torch.float64)
+        self.freq = torch.pow(torch.tensor(self.base, dtype=torch.float64), -2.0 * i / self.width).to(runtime.device).contiguous()
+
+    def emit(self, b, x: int) -> None:
+        from .calls import AddPositionsArgs, emit_library_call
+        if self.freq is None:
+            raise ValueError("the positions have no frequencies laid out (load)")
+        emit_library_call(b, "add_positions", AddPositionsArgs(b._ptr(self.freq), self.width), x)
 
 
 class LMHead(Part):

@@ -65,3 +65,73 @@ class ActivatedMLP(FeedForward):
         self.up.emit(b, src, pre, kernels.EPI_STORE)
         emit_library_call(b, "map_rows", MapRowsArgs(self.ACTIVATIONS[self.activation], self.F, F32, _DT[b.dtype], 0.0), act, inp=pre)
         self.down.emit(b, act, x, kernels.EPI_ACCUMULATE, out_norm=out_norm, out_norm_when=out_norm_when)
+
+
+class RoutedExperts(FeedForward):
+    """A feed-forward of many small gated experts of which every row uses a few:
+        z = W_router h + b;  the `top` largest z pick the experts (ties: the lower index);
+        w = softmax over the picked z alone;  out = sum_k w_k expert_k(h)  (+ shared(h))
+    expert(h) = down(silu(gate h) * (up h)), no biases; `shared_size` > 0 adds one more expert of
+    that inner width that every row passes.  The router's logits, the picks and their weights are
+    float; only the picked experts' weights are read."""
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, prefix: str, hidden_size: int, n_experts: int, top: int, expert_size: int, shared_size: int = 0,
+                 names=("gate", "up", "down")):
+        if not 1 <= top <= n_experts:
+            raise ValueError(f"{top} picks among {n_experts} experts")
+        self.prefix, self.D, self.E, self.top, self.F, self.names = prefix, hidden_size, n_experts, top, expert_size, tuple(names)
+        self.router = Linear([prefix + "router"], [n_experts], hidden_size)
+        self.shared_gate_up = self.shared_down = None
+        if shared_size:
+            self.shared_gate_up = Linear([prefix + "shared." + names[0], prefix + "shared." + names[1]], [shared_size] * 2, hidden_size,
+                                         interleave=True)
+            self.shared_down = Linear([prefix + "shared." + names[2]], [hidden_size], shared_size)
+        self.shared_size = shared_size
+        self.gate = self.up = self.down = self.router_bias = None
+
+    def children(self):
+        return [p for p in (self.router, self.shared_gate_up, self.shared_down) if p is not None]
+
+    def tensor_specs(self):
+        from ..weights import TensorSpec
+        specs = [TensorSpec(self.prefix + "router.b", (self.E,), init="zeros")]
+        for e in range(self.E):
+            p = f"{self.prefix}e{e}."
+            specs += [TensorSpec(p + self.names[0], (self.F, self.D)), TensorSpec(p + self.names[1], (self.F, self.D)),
+                      TensorSpec(p + self.names[2], (self.D, self.F))]
+        return specs
+
+    def load(self, fetch, runtime) -> None:
+        import torch
+
+        def stacked(name):      # [experts][out][in], in the dtype the runtime multiplies in
+            ws = [fetch.get(f"{self.prefix}e{e}.{name}") for e in range(self.E)]
+            if runtime.is_f32 or any(w.dtype == torch.float32 for w in ws):
+                ws = [w.to(torch.float32) for w in ws]
+            return torch.stack(ws, dim=0).contiguous()
+        self.gate, self.up, self.down = (stacked(n) for n in self.names)
+        self.router_bias = fetch.get(self.prefix + "router.b").to(torch.float32).contiguous()
+
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0, accumulate: bool = True) -> None:
+        """x (+)= the picked experts' weighted sum (+ the shared expert) for the rows h of `src`."""
+        import torch
+        from ..engine.program import _DT
+        from .calls import RoutedExpertsArgs, RouteTopArgs, emit_library_call
+        if self.gate is None:
+            raise ValueError(f"the experts of {self.prefix} have no weights loaded")
+        h = b.materialize(src)
+        logits = b.buffer("moe.logits", self.E, torch.float32)
+        self.router.emit(b, h, logits, kernels.EPI_STORE)
+        picks = b.buffer("moe.picks", 2 * self.top, torch.float32)
+        emit_library_call(b, "route_top", RouteTopArgs(b._ptr(self.router_bias), self.E, self.top), picks, inp=logits)
+        written = accumulate
+        if self.shared_size:
+            act = b.buffer("ffn.act", self.shared_size, b.dtype)
+            self.shared_gate_up.emit(b, h, act, kernels.EPI_SWIGLU)
+            self.shared_down.emit(b, act, x, kernels.EPI_ACCUMULATE if accumulate else kernels.EPI_STORE)
+            written = True
+        hidden = b.buffer("moe.hidden", self.top * self.F, torch.float32)
+        args = RoutedExpertsArgs(b._ptr(self.gate), b._ptr(self.up), b._ptr(self.down), _DT[self.gate.dtype], self.E, self.top, self.D,
+                                 self.F, int(written))
+        emit_library_call(b, "routed_experts", args, x, inp=h, extra=[picks, hidden])

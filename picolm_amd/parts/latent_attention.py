@@ -1,0 +1,87 @@
+"""Causal softmax attention whose keys and values are read out of one small latent per token, so
+that only the latent is cached; queries pass a latent of their own; no positions.
+
+    c_q = rms(W_dq h) w_dq;  q = W_uq c_q                       [heads, dim]
+    c   = rms(W_dkv h) w_dkv                                    [kv_rank]: what the cache keeps
+    k_j = W_uk c_j, v_j = W_uv c_j per head;  s_ij = scale (q_i . k_j),  j <= i;  p = softmax(s)
+    out = W_o (concat_heads(sum_j p_ij v_j) * sigmoid(W_g h))
+
+The products with W_uk and W_uv are moved off the cached side: q_i . (W_uk c_j) = (W_uk^T q_i) . c_j
+and sum_j p_ij W_uv c_j = W_uv (sum_j p_ij c_j), so the attention runs over the latents themselves,
+all heads sharing one key head whose keys and values are both c, and a token costs two small
+products per head instead of two per head and cached token.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from ..weights import TensorSpec
+from .base import KVRequest, Mixer, Runtime
+from .calls import GATE_NONE, GATE_SIGMOID, HeadLinearArgs, SinkAttentionArgs, SliceNormArgs, emit_library_call
+from .linear import Linear
+
+
+class LatentAttention(Mixer):
+    graph_safe = True      # launches depend on device memory only
+
+    def __init__(self, prefix: str, hidden_size: int, n_heads: int, head_dim: int, v_head_dim: int, kv_rank: int, q_rank: int,
+                 scale: float, eps: float, gate: bool = True):
+        self.prefix, self.D = prefix, hidden_size
+        self.H, self.d, self.dv, self.r, self.rq = n_heads, head_dim, v_head_dim, kv_rank, q_rank
+        self.scale, self.eps, self.has_gate = float(scale), float(eps), bool(gate)
+        names = [prefix + "dq", prefix + "dkv"] + ([prefix + "g"] if gate else [])
+        self.proj = Linear(names, [q_rank, kv_rank] + ([n_heads * v_head_dim] if gate else []), hidden_size)
+        self.uq = Linear([prefix + "uq"], [n_heads * head_dim], q_rank)
+        self.o = Linear([prefix + "o"], [hidden_size], n_heads * v_head_dim)
+        self.uk = self.uv = self.q_norm = self.c_norm = None
+
+    def children(self):
+        return [self.proj, self.uq, self.o]
+
+    def tensor_specs(self):
+        p = self.prefix
+        return [TensorSpec(p + "dq.norm", (self.rq,), init="ones"), TensorSpec(p + "dkv.norm", (self.r,), init="ones"),
+                TensorSpec(p + "uk", (self.H * self.d, self.r)), TensorSpec(p + "uv", (self.H * self.dv, self.r))]
+
+    def load(self, fetch, runtime: Runtime) -> None:
+        kept = lambda name: (lambda t: t.to(torch.float32) if runtime.is_f32 else t)(fetch.get(self.prefix + name)).contiguous()
+        self.uk, self.uv = kept("uk"), kept("uv")
+        self.q_norm = fetch.get(self.prefix + "dq.norm").to(torch.float32).contiguous()
+        self.c_norm = fetch.get(self.prefix + "dkv.norm").to(torch.float32).contiguous()
+
+    def cache_requests(self):
+        return KVRequest(1, self.r, 0, self.r), None
+
+    def emit(self, b, src, x: int, out_norm=None, out_norm_when: int = 0, accumulate: bool = True) -> None:
+        """x (+)= o(gate * attention) for the rows h of `src`, as operations of a launch program."""
+        from ..engine.program import _DT, F32
+        H, d, dv, r, rq = self.H, self.d, self.dv, self.r, self.rq
+        width = self.proj.out_size
+        engine_dt = _DT[b.dtype]
+        rows = b.buffer("latent.in", width, torch.float32)
+        self.proj.emit(b, src, rows, kernels.EPI_STORE)
+        cq = b.buffer("latent.cq", rq, b.dtype)
+        emit_library_call(b, "slice_norm", SliceNormArgs(b._ptr(self.q_norm), rq, width, 0, rq, 0, engine_dt, self.eps), cq, inp=rows)
+        q = b.buffer("latent.q", H * d, torch.float32)
+        self.uq.emit(b, cq, q, kernels.EPI_STORE)
+        # [W_uk^T q per head | c]: the attention's queries, and its one key and value
+        qc = b.buffer("latent.qc", H * r + r, torch.float32)
+        weight_dt = _DT[self.uk.dtype]
+        emit_library_call(b, "head_linear", HeadLinearArgs(b._ptr(self.uk), weight_dt, H, d, r, 1, H * d, 0, F32, H * r + r, 0, F32,
+                                                           GATE_NONE, 0, 0), qc, inp=q)
+        emit_library_call(b, "slice_norm", SliceNormArgs(b._ptr(self.c_norm), r, width, rq, H * r + r, H * r, F32, self.eps), qc, inp=rows)
+        scratch = b.buffer("latent.q.rows", H * r, b.dtype)
+        att = b.buffer("latent.att", H * r, b.dtype)
+        args = SinkAttentionArgs(H, 1, r, r, H * r + r, 0, H * r, H * r, -1, self.scale, self.eps, None, None, None, 0, None)
+        lib = kernels.lib()
+        on_matrix_cores = b.dtype == torch.bfloat16 and lib.picolm_attn_plain_mfma_takes(r, r)
+        emit_library_call(b, "sink_attention", args, att, inp=qc, extra=[scratch], uses_kv=True, attends=True,
+                          tile_rows=lib.picolm_attn_plain_mfma_tile_rows() if on_matrix_cores else kernels.attn_prefill_tile_rows(),
+                          partial_floats=H * (r + 2))
+        heads = b.buffer("latent.heads", H * dv, b.dtype)
+        emit_library_call(b, "head_linear", HeadLinearArgs(b._ptr(self.uv), weight_dt, H, r, dv, 0, H * r, 0, engine_dt, H * dv, 0, engine_dt,
+                                                           GATE_SIGMOID if self.has_gate else GATE_NONE, width, rq + r), heads, inp=att,
+                          extra=[rows] if self.has_gate else [])
+        self.o.emit(b, heads, x, kernels.EPI_ACCUMULATE if accumulate else kernels.EPI_STORE,
+                    **({"out_norm": out_norm, "out_norm_when": out_norm_when} if accumulate else {}))
