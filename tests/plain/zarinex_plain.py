@@ -135,29 +135,41 @@ def routed_experts(h, W, p, mlp):
     return out
 
 
+def router_margins(h, W, p, mlp):
+    """Per row, how far the last picked logit lies above the first one that is not picked (inf where
+    every expert is picked): a row with a small margin may pick otherwise after a rounding."""
+    E, top = mlp["router"]["experts"], mlp["router"]["top"]
+    if top >= E:
+        return np.full(h.shape[0], np.inf)
+    z = -np.sort(-(h @ W[p + "router"].T + W[p + "router.b"]), axis=1)
+    return z[:, top - 1] - z[:, top]
+
+
 MIXERS = {"mamba1": lambda h, W, p, m, eps: mamba1(h, W, p, m), "latent_attention": latent_attention, "hgrn2": hgrn2}
 
 
-def layer(x, W, p, entry, alpha, eps):
+def layer(x, W, p, entry, alpha, eps, margins=None):
     u = MIXERS[entry["type"]](token_shift(x, W[p + "shift"]), W, p + "mix.", entry["mixer"], eps)
     u = u * sigmoid(x @ W[p + "rg1"].T + W[p + "rg1.b"])
     x = rms_norm(alpha * x + u, W[p + "norm1"], eps)
     if entry.get("mlp"):
+        if margins is not None:
+            margins.append(router_margins(x, W, p + "mlp.", entry["mlp"]))
         u = routed_experts(x, W, p + "mlp.", entry["mlp"]) * sigmoid(x @ W[p + "rg2"].T + W[p + "rg2.b"])
         x = rms_norm(alpha * x + u, W[p + "norm2"], eps)
     return x
 
 
-def forward(config: dict, W: dict, tokens, return_layers: bool = False):
+def forward(config: dict, W: dict, tokens, return_layers: bool = False, margins: list | None = None):
     """logits [T, vocab] of one sequence from its first token; with return_layers also the rows
-    after every layer run."""
+    after every layer run; `margins` collects every routed layer run's margins per row."""
     W = {k: np.asarray(v, np.float64) for k, v in W.items()}
     D, eps, alpha = config["width"], config["norm"]["eps"], config["postln_alpha"]
     x = W["embed"][np.asarray(tokens)] + position_rows(range(len(tokens)), D)
     after = []
     for i, entry in enumerate(config["layers"]):
         owner = entry.get("weights_of")
-        x = layer(x, W, f"l{i if owner is None else owner}.", entry, alpha, eps)
+        x = layer(x, W, f"l{i if owner is None else owner}.", entry, alpha, eps, margins)
         after.append(x)
     logits = rms_norm(x, W["final.norm"], eps) @ W["embed"].T
     return (logits, np.stack(after)) if return_layers else logits

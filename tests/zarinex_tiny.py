@@ -155,7 +155,37 @@ def plain_logits(cfg: dict, weights: dict, tokens) -> np.ndarray:
     return P.forward(cfg, {k: v.to(torch.float64).numpy() for k, v in weights.items()}, list(tokens))
 
 
+class Truth:
+    """The plain model's logits of a sequence, and per token the smallest margin by which any of
+    its routers picked."""
+
+    def __init__(self, cfg: dict, weights: dict, tokens):
+        from plain import zarinex_plain as P
+        margins = []
+        self.logits = P.forward(cfg, {k: v.to(torch.float64).numpy() for k, v in weights.items()}, list(tokens), margins=margins)
+        self.margins = np.min(margins, axis=0) if margins else np.full(len(tokens), np.inf)
+
+    def __getitem__(self, rows):
+        return self.logits[rows]
+
+
+def near(got, truth: Truth, rows, dtype: str) -> bool:
+    """Whether the engine's rows lie within the limit of the plain model's.  A token whose router
+    picked by less than CLOSE_CALL is held to LOOSE instead: rounding may give it another expert, and
+    then its row is another function's value."""
+    rows = np.arange(len(truth.logits))[rows]
+    got, want = np.atleast_2d(np.asarray(got, np.float64)), np.atleast_2d(truth.logits[rows])
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    spread = np.sqrt(((want - want.mean(-1, keepdims=True)) ** 2).mean())
+    e = np.sqrt((d ** 2).mean(-1)) / spread
+    limit = np.where(np.atleast_1d(truth.margins[rows]) < CLOSE_CALL[dtype], LOOSE, LIMIT[dtype])
+    return bool((e <= limit).all())
+
+
 # in 32-bit the engine's sums differ from the plain model's double precision by rounding alone; in
 # bfloat16 every product's input is rounded to eight bits, and a router's logits that lie close
 # together may then pick another expert for a token
 LIMIT = {"float32": 2e-4, "bfloat16": 0.08}
+CLOSE_CALL = {"float32": 1e-4, "bfloat16": 0.1}      # router logits have a spread of about two
+LOOSE = 0.5
