@@ -171,15 +171,18 @@ class Truth:
 
 def near(got, truth: Truth, rows, dtype: str) -> bool:
     """Whether the engine's rows lie within the limit of the plain model's.  A token whose router
-    picked by less than CLOSE_CALL is held to LOOSE instead: rounding may give it another expert, and
-    then its row is another function's value."""
+    picked by less than CLOSE_CALL is held to LOOSE instead, and so are the AFTER tokens behind it:
+    rounding may give it another expert, and then its row is another function's value, which the
+    next tokens read through the blend, the convolution and the states."""
     rows = np.arange(len(truth.logits))[rows]
     got, want = np.atleast_2d(np.asarray(got, np.float64)), np.atleast_2d(truth.logits[rows])
     d = got - want
     d = d - d.mean(-1, keepdims=True)
     spread = np.sqrt(((want - want.mean(-1, keepdims=True)) ** 2).mean())
     e = np.sqrt((d ** 2).mean(-1)) / spread
-    limit = np.where(np.atleast_1d(truth.margins[rows]) < CLOSE_CALL[dtype], LOOSE, LIMIT[dtype])
+    close = truth.margins < CLOSE_CALL[dtype]
+    shaky = np.array([close[max(0, r - AFTER):r + 1].any() for r in np.atleast_1d(rows)])
+    limit = np.where(shaky, LOOSE, LIMIT[dtype])
     return bool((e <= limit).all())
 
 
@@ -187,5 +190,5 @@ def near(got, truth: Truth, rows, dtype: str) -> bool:
 # bfloat16 every product's input is rounded to eight bits, and a router's logits that lie close
 # together may then pick another expert for a token
 LIMIT = {"float32": 2e-4, "bfloat16": 0.08}
-CLOSE_CALL = {"float32": 1e-4, "bfloat16": 0.1}      # router logits have a spread of about two
-LOOSE = 0.5
+CLOSE_CALL = {"float32": 1e-4, "bfloat16": 0.03}     # router logits have a spread of about two
+LOOSE, AFTER = 0.5, 6
