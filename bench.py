@@ -177,12 +177,6 @@ def _begopel_pair(width: int, heads: int, kv_heads: int, ff: int, vocab: int, pa
     return beg, llama
 
 
-DESIGN_SIZES = {
-    "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
-                ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
-}
-
-
 def _begopel_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
     """Per label of operation, the seconds that the work of one prefill step of T tokens and of one
     decode step of n_seq sequences at `context` would take at the peak that binds it: products and
@@ -210,13 +204,69 @@ def _begopel_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
     return {"prefill": pre, "decode": dec}
 
 
+def _zarinex_pair(width: int, heads: int, kv_rank: int, experts: int, top: int, vocab: int, runs: int):
+    """A Zarinex of `runs` layers in the order (hgrn2, mamba1, latent attention, mamba1) with heads of
+    128, a selective scan of twice the width with a state of 16, and `experts` experts as wide as the
+    model of which a token uses `top` beside a shared one; and the Begopel of the same width, heads,
+    vocabulary and number of layer runs whose dense feed-forward is as wide as the experts a token uses."""
+    mlp = dict(kind="moe", router=dict(experts=experts, top=top), expert=dict(ff=width), shared=dict(ff=width))
+    kinds = [("hgrn2", dict(heads=heads, dim=128, vdim=128)),
+             ("mamba1", dict(inner=2 * width, state=16, dt_rank=width // 16, conv=4)),
+             ("latent_attention", dict(heads=heads, dim=128, vdim=128, kv_rank=kv_rank, q_rank=3 * kv_rank, scale=128 ** -0.5)),
+             ("mamba1", dict(inner=2 * width, state=16, dt_rank=width // 16, conv=4))]
+    if runs < 4:
+        kinds = kinds[1:3]
+    layers = [dict(type=t, mixer=m, mlp=mlp) for t, m in kinds[:runs]]
+    zar = dict(architecture="Zarinex", vocab=vocab, width=width, norm=dict(eps=1e-6), postln_alpha=1.0, layers=layers)
+    beg, _ = _begopel_pair(width, heads, max(heads // 4, 1), (top + 1) * width, vocab, runs // 2)
+    return zar, beg
+
+
+DESIGN_SIZES = {
+    "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
+                ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
+    "zarinex": [("width 1024", (1024, 8, 128, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 128, 8, 2, 32000, 4)),
+                ("width 4096, latents of 512", (4096, 32, 512, 16, 2, 128256, 2))],
+}
+
+
+def _zarinex_rooflines(cfg: dict, T: int, n_seq: int, context: int) -> dict:
+    """As _begopel_rooflines, for the operations of a Zarinex: the attention over latents (keys and
+    values are both the latent) at the bf16 matrix peak, the walk of the states at the 32-bit vector
+    peak (6 flops per state element and token with a decay per element, 5 with one per row), the
+    picked experts' products at the bf16 matrix peak; in a decode step the latents twice (the cache
+    keeps them in the keys' and in the values' layout), twice the states, and the weights of the
+    experts that the step's tokens can pick at most, at HBM's peak."""
+    mfma, valu, hbm = PEAK_TFLOPS["bf16"] * 1e12, PEAK_TFLOPS["fp32"] * 1e12, HBM_PEAK_GBS * 1e9
+    names = ("sink_attention", "decay_scan", "routed_experts")
+    pre, dec = {k: 0.0 for k in names}, {k: 0.0 for k in names}
+    D = cfg["width"]
+    for layer in cfg["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "latent_attention":
+            pre["sink_attention"] += 2.0 * m["heads"] * 2 * m["kv_rank"] * (T * (T + 1) / 2) / mfma
+            dec["sink_attention"] += n_seq * context * 2 * m["kv_rank"] * 2 / hbm
+        elif layer["type"] == "mamba1":
+            pre["decay_scan"] += 6.0 * T * m["inner"] * m["state"] / valu
+            dec["decay_scan"] += n_seq * 2 * m["inner"] * m["state"] * 4 / hbm
+        else:
+            pre["decay_scan"] += 5.0 * T * m["heads"] * m["dim"] * m["vdim"] / valu
+            dec["decay_scan"] += n_seq * 2 * m["heads"] * m["dim"] * m["vdim"] * 4 / hbm
+        mlp = layer.get("mlp")
+        if mlp:
+            E, top, F = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["ff"]
+            pre["routed_experts"] += 2.0 * 3 * T * top * D * F / mfma
+            dec["routed_experts"] += min(n_seq * top, E) * 3 * D * F * 2 / hbm
+    return {"prefill": pre, "decode": dec}
+
+
 def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int) -> dict:
     """Prefill and decode throughput of `design` at a few sizes that resemble real layers (random
-    weights), beside the Llama of equal size, and the GPU time of one prefill step and one decode
-    step by operation."""
+    weights), beside the closest model the library has at equal size (for Begopel the Llama, for
+    Zarinex the Begopel), and the GPU time of one prefill step and one decode step by operation."""
     import torch
 
-    from picolm_amd.config import BegopelConfig, LlamaConfig
+    from picolm_amd.config import LlamaConfig, resolve
     from picolm_amd.engine import Session, random_model
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(0)
@@ -267,19 +317,28 @@ def design_comparison(design: str, T: int, n_seq: int, context: int, steps: int)
         torch.cuda.empty_cache()
         return res
 
+    def fractions_of(roof, res):
+        return {phase: {k: roof[phase][k] / (res[phase + "_ops_ms"][k] * 1e-3) for k in roof[phase] if res[phase + "_ops_ms"].get(k)}
+                for phase in ("prefill", "decode")}
+
     for name, size in DESIGN_SIZES[design]:
-        beg, llama = _begopel_pair(*size)
         print(f"[bench] {design} {name}", file=sys.stderr, flush=True)
-        a = measure(BegopelConfig.from_dict(beg), beg["vocab"])
+        if design == "zarinex":
+            zar, beg = _zarinex_pair(*size)
+            a = measure(resolve(zar).parse_config(zar), zar["vocab"])
+            b = measure(resolve(beg).parse_config(beg), beg["vocab"])
+            out["sizes"].append({"size": name, "layer_runs": len(zar["layers"]), design: a, "begopel": b,
+                                 "fraction_of_roofline": fractions_of(_zarinex_rooflines(zar, T, n_seq, context), a),
+                                 "begopel_fraction_of_roofline": fractions_of(_begopel_rooflines(beg, T, n_seq, context), b)})
+            continue
+        beg, llama = _begopel_pair(*size)
+        a = measure(resolve(beg).parse_config(beg), beg["vocab"])
         b = measure(LlamaConfig.from_dict(llama), llama["vocab_size"])
-        roof = _begopel_rooflines(beg, T, n_seq, context)
         lc = LlamaConfig.from_dict(llama)
         like = {"prefill": attention_flops(lc, T) / (PEAK_TFLOPS["bf16"] * 1e12),
                 "decode": n_seq * context * kv_bytes_per_token(lc) / (HBM_PEAK_GBS * 1e9)}
-        fractions = {}
+        fractions = fractions_of(_begopel_rooflines(beg, T, n_seq, context), a)
         for phase in ("prefill", "decode"):
-            ops = a[phase + "_ops_ms"]
-            fractions[phase] = {k: roof[phase][k] / (ops[k] * 1e-3) for k in roof[phase] if ops.get(k)}
             fractions[phase]["llama attention"] = like[phase] / (b[phase + "_ops_ms"]["attention"] * 1e-3)
         out["sizes"].append({"size": name, "layer_runs": llama["num_hidden_layers"], design: a, "llama": b,
                              "fraction_of_roofline": fractions})

@@ -238,7 +238,9 @@ int picolm_call_route_top(void* user, const picolm_step_view* v);
 // The picked experts of every row: y[t][k] = W_down[e] (silu(W_gate[e] h) * (W_up[e] h)), e the k-th
 // pick of row t, and their weighted sum  out[t] = sum_k w[t][k] y[t][k] (+ out[t] if `adds`).
 //   in: h rows [width] in the engine's dtype; extra[0]: the picks as route_top leaves them; extra[1]:
-//   scratch float rows [top width]; out: float rows [width].
+//   scratch float rows [top ff]; out: float rows [width].  With extra[2], scratch float rows
+//   [top width], and extra[3], scratch rows of top + experts + 1 words, a step of many rows in
+//   bfloat16 sorts its (row, pick) pairs by expert and runs them through the matrix cores.
 typedef struct {
     const void* gate;        // [experts][ff][width]
     const void* up;          // [experts][ff][width]

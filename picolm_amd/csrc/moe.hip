@@ -4,10 +4,17 @@
 // workgroup per (row, 16 outputs)), so that a row's result is added up in one place and in a fixed
 // order.  A wave takes one weight row at a time, 16 bytes a lane, against the row's input in LDS.
 // Logits, picks, weights, hidden units and sums are float.
+//
+// A prompt (64 rows and more, bfloat16) goes through the matrix cores instead: the (row, pick) pairs
+// are sorted by expert in one workgroup, a wave takes 32 pairs of one expert by 32 hidden units (or
+// outputs) with v_mfma_f32_32x32x16_bf16, its operands straight from global memory, 16 bytes a
+// lane; the hidden units are rounded to bfloat16 once, as every product's input is; a last kernel
+// adds a row's picks up in their order.  Which pairs share a tile changes no pair's result.
 #include "mixers.h"
 
 #include "api.h"
 #include "common.h"
+#include "gemm_mfma.h"
 
 #define VIEW_REQUIRE(who, v)                                                                                      \
     PICOLM_REQUIRE((v) && (v)->struct_bytes == (int32_t)sizeof(picolm_step_view), "%s: the step view is of another version", who)
@@ -134,6 +141,133 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restric
     }
 }
 
+// ---- the same for many rows, on the matrix cores ------------------------------------------------------
+#define GM_ROWS 32       // pairs of a tile
+#define GM_MAX_EXPERTS 4096
+
+// plan: [0 .. E] where each expert's pairs start in the sorted list, then the sorted pairs (pair = row * top + pick)
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ picks, int32_t* __restrict__ plan, int E, int top,
+                                                        int n_pairs) {
+    extern __shared__ int32_t plan_lds[];      // counts, then cursors [E] | starts [E + 1]
+    int32_t* counts = plan_lds;
+    int32_t* starts = plan_lds + E;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = picks[(size_t)(p / top) * 2 * top + p % top];
+        if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < E; ++e) {
+            starts[e] = at;
+            at += counts[e];
+            counts[e] = 0;
+        }
+        starts[E] = at;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e <= E; e += blockDim.x) plan[e] = starts[e];
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = picks[(size_t)(p / top) * 2 * top + p % top];
+        if (e >= 0 && e < E) plan[E + 1 + starts[e] + atomicAdd(&counts[e], 1)] = p;
+    }
+}
+
+// the tile of GM_ROWS pairs that a workgroup takes: its expert, and its pairs into LDS (-1 past the expert's last)
+__device__ __forceinline__ int tile_of(const int32_t* __restrict__ plan, int E, int tile, int32_t* pairs_lds) {
+    int e = 0, first = 0;
+    for (; e < E; ++e) {
+        const int n = plan[e + 1] - plan[e], tiles = (n + GM_ROWS - 1) / GM_ROWS;
+        if (tile < tiles) {
+            first = plan[e] + tile * GM_ROWS;
+            break;
+        }
+        tile -= tiles;
+    }
+    if (e == E) return -1;
+    if (threadIdx.x < GM_ROWS) pairs_lds[threadIdx.x] = first + (int)threadIdx.x < plan[e + 1] ? plan[E + 1 + first + threadIdx.x] : -1;
+    __syncthreads();
+    return e;
+}
+
+// act[pair][f] = bf16(silu(gate[e][f] . h[row]) * (up[e][f] . h[row])); a wave takes 32 pairs by 32 hidden units
+__global__ __launch_bounds__(256) void grouped_hidden_kernel(const bf16_t* __restrict__ h, const int32_t* __restrict__ plan, bf16_t* __restrict__ act,
+                                                             const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up, int E, int top, int D,
+                                                             int F) {
+    __shared__ int32_t pairs[GM_ROWS];
+    const int e = tile_of(plan, E, blockIdx.x, pairs);
+    if (e < 0) return;
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, l32 = lane % 32, kq = lane / 32;
+    const int f0 = (blockIdx.y * 4 + wave) * 32;
+    if (f0 >= F) return;
+    const int my_pair = pairs[l32];
+    const bf16_t* a_row = h + (size_t)(my_pair >= 0 ? my_pair / top : 0) * D + kq * 8;
+    const size_t w_row = ((size_t)e * F + min(f0 + l32, F - 1)) * D + kq * 8;
+    const bf16_t* g_row = gate + w_row;
+    const bf16_t* u_row = up + w_row;
+    f32x16 acc_g, acc_u;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc_g[i] = acc_u[i] = 0.f;
+#pragma unroll 4
+    for (int k = 0; k < D; k += 16) {
+        const bf16x8 a = my_pair >= 0 ? load_chunk(a_row + k) : zero_chunk();
+        acc_g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(g_row + k), acc_g, 0, 0, 0);
+        acc_u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(u_row + k), acc_u, 0, 0, 0);
+    }
+    if (f0 + l32 >= F) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int pair = pairs[8 * (i / 4) + i % 4 + 4 * kq];
+        if (pair >= 0) act[(size_t)pair * F + f0 + l32] = f32_to_bf16_bits(acc_g[i] / (1.f + expf(-acc_g[i])) * acc_u[i]);
+    }
+}
+
+// y[pair][d] = down[e][d] . act[pair]; a wave takes 32 pairs by 32 outputs
+__global__ __launch_bounds__(256) void grouped_down_kernel(const bf16_t* __restrict__ act, const int32_t* __restrict__ plan, float* __restrict__ y,
+                                                           const bf16_t* __restrict__ down, int E, int D, int F) {
+    __shared__ int32_t pairs[GM_ROWS];
+    const int e = tile_of(plan, E, blockIdx.x, pairs);
+    if (e < 0) return;
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, l32 = lane % 32, kq = lane / 32;
+    const int d0 = (blockIdx.y * 4 + wave) * 32;
+    if (d0 >= D) return;
+    const int my_pair = pairs[l32];
+    const bf16_t* a_row = act + (size_t)max(my_pair, 0) * F + kq * 8;
+    const bf16_t* w_row = down + ((size_t)e * D + min(d0 + l32, D - 1)) * F + kq * 8;
+    f32x16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll 4
+    for (int k = 0; k < F; k += 16) {
+        const bf16x8 a = my_pair >= 0 ? load_chunk(a_row + k) : zero_chunk();
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(w_row + k), acc, 0, 0, 0);
+    }
+    if (d0 + l32 >= D) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int pair = pairs[8 * (i / 4) + i % 4 + 4 * kq];
+        if (pair >= 0) y[(size_t)pair * D + d0 + l32] = acc[i];
+    }
+}
+
+// out[row] (+)= sum_k w[row][k] y[row][k], in the order of the picks
+__global__ void grouped_sum_kernel(const float* __restrict__ y, const int32_t* __restrict__ picks, float* __restrict__ out, int E, int top, int D,
+                                   int adds) {
+    const size_t row = blockIdx.x;
+    const int32_t* ids = picks + row * 2 * top;
+    const float* w = (const float*)(ids + top);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float total = 0.f;
+        for (int k = 0; k < top; ++k)
+            if (ids[k] >= 0 && ids[k] < E) total += w[k] * y[(row * top + k) * D + d];
+        out[row * D + d] = (adds ? out[row * D + d] : 0.f) + total;
+    }
+}
+
+#define GM_FROM_ROWS 64      // rows of a step from which the matrix cores take the experts
+
 extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v) {
     const picolm_routed_experts_args* a = (const picolm_routed_experts_args*)user;
     VIEW_REQUIRE("routed_experts", v);
@@ -153,6 +287,25 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
     if (v->rows <= 0) return 0;
     const int32_t* picks = (const int32_t*)v->extra[0];
     float* act = (float*)v->extra[1];
+    if (v->dtype == PICOLM_BF16 && a->weight_dt == PICOLM_BF16 && v->rows >= GM_FROM_ROWS && D % 16 == 0 && F % 16 == 0 && E <= GM_MAX_EXPERTS &&
+        v->extra[2] && v->extra[3]) {
+        const int64_t n_pairs = (int64_t)v->rows * top;
+        PICOLM_REQUIRE(v->extra_row_bytes[2] >= (int64_t)top * D * 4 && v->extra_row_bytes[3] >= (int64_t)(top + E + 1) * 4,
+                       "routed_experts: scratch rows too short for the sorted pairs or their outputs");
+        int32_t* plan = (int32_t*)v->extra[3];
+        float* y = (float*)v->extra[2];
+        moe_plan_kernel<<<1, 1024, sizeof(int32_t) * (2 * (size_t)E + 1), v->stream>>>(picks, plan, E, top, (int)n_pairs);
+        PICOLM_LAUNCH_CHECK("routed_experts (plan)");
+        const unsigned tiles = (unsigned)(ceil_div64(n_pairs, GM_ROWS) + E);      // no more than these are filled; the rest leave at once
+        grouped_hidden_kernel<<<dim3(tiles, ceil_div(F, 128)), 256, 0, v->stream>>>((const bf16_t*)v->in, plan, (bf16_t*)act, (const bf16_t*)a->gate,
+                                                                                   (const bf16_t*)a->up, E, top, D, F);
+        PICOLM_LAUNCH_CHECK("routed_experts (hidden, grouped)");
+        grouped_down_kernel<<<dim3(tiles, ceil_div(D, 128)), 256, 0, v->stream>>>((const bf16_t*)act, plan, y, (const bf16_t*)a->down, E, D, F);
+        PICOLM_LAUNCH_CHECK("routed_experts (down, grouped)");
+        grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds);
+        PICOLM_LAUNCH_CHECK("routed_experts (sum)");
+        return 0;
+    }
     const dim3 grid_a((unsigned)(v->rows * top), ceil_div(F, MOE_UNITS)), grid_b(v->rows, ceil_div(D, MOE_UNITS));
     if (a->weight_dt == PICOLM_F32 && v->dtype == PICOLM_F32) {
         expert_hidden_kernel<float, float><<<grid_a, 256, lds_a, v->stream>>>((const float*)v->in, picks, act, (const float*)a->gate,

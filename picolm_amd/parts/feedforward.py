@@ -134,4 +134,6 @@ class RoutedExperts(FeedForward):
         hidden = b.buffer("moe.hidden", self.top * self.F, torch.float32)
         args = RoutedExpertsArgs(b._ptr(self.gate), b._ptr(self.up), b._ptr(self.down), _DT[self.gate.dtype], self.E, self.top, self.D,
                                  self.F, int(written))
-        emit_library_call(b, "routed_experts", args, x, inp=h, extra=[picks, hidden])
+        pair_out = b.buffer("moe.pairs", self.top * self.D, torch.float32)
+        plan = b.buffer("moe.plan", self.top + self.E + 1, torch.float32)
+        emit_library_call(b, "routed_experts", args, x, inp=h, extra=[picks, hidden, pair_out, plan])

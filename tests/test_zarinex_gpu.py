@@ -88,6 +88,10 @@ ALONE = {
     "routed experts": one_layer(zt.hgrn(1, 8, 8), zt.moe(6, 2, 24, 40)),
     "routed experts, one pick, no shared expert": one_layer(zt.hgrn(1, 8, 8), zt.moe(5, 1, 36)),
     "routed experts, every expert picked": one_layer(zt.hgrn(1, 8, 8), zt.moe(3, 3, 20, 12)),
+    # in bfloat16 a prompt of 64 rows and more sorts its picks by expert for the matrix cores: tiles that are partly
+    # empty, experts without a row, hidden units and outputs that end inside a tile of 32
+    "routed experts, widths in multiples of 16": one_layer(zt.hgrn(1, 8, 8), zt.moe(6, 2, 32, 48)),
+    "routed experts, more experts than rows a tile": one_layer(zt.hgrn(1, 8, 8), zt.moe(40, 3, 48)),
     "routed experts, widths that are no multiples of 8": zt.config(61, 45, [zt.layer(zt.hgrn(1, 9, 5), zt.moe(4, 2, 13, 7))]),
     "alpha and eps": one_layer(zt.hgrn(2, 8, 12), zt.moe(2, 1, 16, 8), alpha=5.0, eps=1e-2),
 }
