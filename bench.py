@@ -226,7 +226,7 @@ DESIGN_SIZES = {
     "begopel": [("width 1024", (1024, 8, 2, 4096, 32000, 2, 2)), ("width 2048", (2048, 16, 4, 8192, 32000, 2, 0)),
                 ("width 4096", (4096, 32, 8, 14336, 128256, 1, 0))],
     "zarinex": [("width 1024", (1024, 8, 128, 8, 2, 32000, 4)), ("width 2048", (2048, 16, 128, 8, 2, 32000, 4)),
-                ("width 4096, latents of 512", (4096, 32, 512, 16, 2, 128256, 2))],
+                ("width 4096", (4096, 32, 128, 16, 2, 128256, 2)), ("width 4096, latents of 512", (4096, 32, 512, 16, 2, 128256, 2))],
 }
 
 

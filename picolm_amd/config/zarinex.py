@@ -54,6 +54,8 @@ class LatentAttentionConfig:
     def from_dict(d: dict, where: str) -> "LatentAttentionConfig":
         c = LatentAttentionConfig(_integer(d, where, "heads"), _integer(d, where, "dim"), _integer(d, where, "vdim"),
                                   _integer(d, where, "kv_rank"), _integer(d, where, "q_rank"), _number(d, where, "scale"))
+        if not c.scale > 0:
+            raise ConfigError(f"{where}scale: must be positive")
         if c.kv_rank > MAX_HEAD_DIM:        # the attention runs over the latents: they are its keys
             raise ConfigError(f"{where}kv_rank: {c.kv_rank} exceeds {MAX_HEAD_DIM}, the largest key the attention kernels take")
         return c
@@ -178,11 +180,14 @@ class ZarinexConfig:
         if self.torch_dtype not in ("bfloat16", "float32", "float16"):
             raise ConfigError(f"torch_dtype: '{self.torch_dtype}' is not one of bfloat16, float32, float16")
         for i, layer in enumerate(self.layers):
-            j = layer.weights_of
-            if j is None:
+            if layer.weights_of is None:
                 continue
-            if not 0 <= j < len(self.layers) or j == i or self.layers[j].weights_of is not None:
-                raise ConfigError(f"layers[{i}].weights_of: {j} is no other layer with tensors of its own")
+            j, seen = i, set()
+            while self.layers[j].weights_of is not None:       # a layer may name one that names another
+                seen.add(j)
+                j = self.layers[j].weights_of
+                if not 0 <= j < len(self.layers) or j in seen:
+                    raise ConfigError(f"layers[{i}].weights_of: {layer.weights_of} leads to no layer with tensors of its own")
             owner = self.layers[j]
             if (owner.type, owner.mixer, owner.mlp) != (layer.type, layer.mixer, layer.mlp):
                 raise ConfigError(f"layers[{i}].weights_of: layer {j} has other sizes than this one")
@@ -212,5 +217,6 @@ class ZarinexConfig:
 
     def owner_of(self, i: int) -> int:
         """The layer whose tensors layer i runs with."""
-        j = self.layers[i].weights_of
-        return i if j is None else j
+        while self.layers[i].weights_of is not None:
+            i = self.layers[i].weights_of
+        return i

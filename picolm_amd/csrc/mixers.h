@@ -182,7 +182,8 @@ int picolm_call_head_linear(void* user, const picolm_step_view* v);
 
 // The sum and the norm of a layer that norms after adding:
 //   x <- (alpha x + u act(g + bias)) / rms(.) * weight          act = sigmoid where g is given, 1 else
-//   out: x float rows [width]; in: u float rows [width]; extra[0] (optional): g float rows [width].
+//   out: x float rows [width]; in: u float rows [width]; extra[0] (optional): g float rows [width];
+//   extra[1] (optional): the new x once more, in the engine's dtype, for the products that read it next.
 typedef struct {
     const float* weight;     // [width]
     const float* gate_bias;  // [width] or null

@@ -6,10 +6,10 @@
 // Logits, picks, weights, hidden units and sums are float.
 //
 // A prompt (64 rows and more, bfloat16) goes through the matrix cores instead: the (row, pick) pairs
-// are sorted by expert in one workgroup, a wave takes 32 pairs of one expert by 32 hidden units (or
-// outputs) with v_mfma_f32_32x32x16_bf16, its operands straight from global memory, 16 bytes a
-// lane; the hidden units are rounded to bfloat16 once, as every product's input is; a last kernel
-// adds a row's picks up in their order.  Which pairs share a tile changes no pair's result.
+// are sorted by expert in one workgroup, a workgroup takes 128 pairs of one expert by 64 hidden units
+// (or outputs) through LDS with v_mfma_f32_32x32x16_bf16; the hidden units are rounded to bfloat16
+// once, as every product's input is; a last kernel adds a row's picks up in their order.  Which
+// pairs share a tile changes no pair's result.
 #include "mixers.h"
 
 #include "api.h"
@@ -98,7 +98,7 @@ template <> __device__ __forceinline__ float lane_dot<float>(const float* __rest
 
 #define MOE_UNITS 16     // hidden units, or outputs, a workgroup of four waves takes
 
-// act[row][pick][f] = silu(W_gate[e][f] . h) * (W_up[e][f] . h)
+// act[row][pick][f] = silu(W_gate[e][f] . h) * (W_up[e][f] . h); a wave has its four units' eight rows on their way at once
 template <typename TW, typename TH>
 __global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict__ h, const int32_t* __restrict__ picks, float* __restrict__ act,
                                                             const TW* __restrict__ gate, const TW* __restrict__ up, int E, int top, int D, int F) {
@@ -109,12 +109,18 @@ __global__ __launch_bounds__(256) void expert_hidden_kernel(const TH* __restrict
     __syncthreads();
     if (e < 0 || e >= E) return;
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int f1 = min(F, (int)(blockIdx.y + 1) * MOE_UNITS);
-    for (int f = blockIdx.y * MOE_UNITS + wave; f < f1; f += blockDim.x / WAVE) {
-        const size_t w_row = ((size_t)e * F + f) * D;
-        const float g = wave_sum(lane_dot<TW>(gate + w_row, moe_lds, D, lane));
-        const float u = wave_sum(lane_dot<TW>(up + w_row, moe_lds, D, lane));
-        if (lane == 0) act[((size_t)row * top + k) * F + f] = g / (1.f + expf(-g)) * u;
+    const int f0 = blockIdx.y * MOE_UNITS + wave * 4;
+    float g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const size_t w_row = ((size_t)e * F + min(f0 + j, F - 1)) * D;
+        g[j] = lane_dot<TW>(gate + w_row, moe_lds, D, lane);
+        u[j] = lane_dot<TW>(up + w_row, moe_lds, D, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float gs = wave_sum(g[j]), us = wave_sum(u[j]);
+        if (lane == 0 && f0 + j < F) act[((size_t)row * top + k) * F + f0 + j] = gs / (1.f + expf(-gs)) * us;
     }
 }
 
@@ -129,20 +135,24 @@ __global__ __launch_bounds__(256) void expert_down_kernel(const float* __restric
     const int32_t* ids = picks + (size_t)row * 2 * top;
     const float* w = (const float*)(ids + top);
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int d1 = min(D, (int)(blockIdx.y + 1) * MOE_UNITS);
-    for (int d = blockIdx.y * MOE_UNITS + wave; d < d1; d += blockDim.x / WAVE) {
-        float total = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int e = ids[k];
-            if (e < 0 || e >= E) continue;
-            total += w[k] * wave_sum(lane_dot<TW>(down + ((size_t)e * D + d) * F, moe_lds + (size_t)k * F, F, lane));
-        }
-        if (lane == 0) out[(size_t)row * D + d] = (adds ? out[(size_t)row * D + d] : 0.f) + total;
+    const int d0 = blockIdx.y * MOE_UNITS + wave * 4;
+    float total[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < top; ++k) {
+        const int e = ids[k];
+        if (e < 0 || e >= E) continue;
+        float part[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) part[j] = lane_dot<TW>(down + ((size_t)e * D + min(d0 + j, D - 1)) * F, moe_lds + (size_t)k * F, F, lane);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) total[j] += w[k] * wave_sum(part[j]);
     }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (lane == 0 && d0 + j < D) out[(size_t)row * D + d0 + j] = (adds ? out[(size_t)row * D + d0 + j] : 0.f) + total[j];
 }
 
 // ---- the same for many rows, on the matrix cores ------------------------------------------------------
-#define GM_ROWS 32       // pairs of a tile
+#define GM_ROWS 128      // pairs of a tile
 #define GM_MAX_EXPERTS 4096
 
 // plan: [0 .. E] where each expert's pairs start in the sorted list, then the sorted pairs (pair = row * top + pick)
@@ -187,69 +197,96 @@ __device__ __forceinline__ int tile_of(const int32_t* __restrict__ plan, int E, 
         tile -= tiles;
     }
     if (e == E) return -1;
-    if (threadIdx.x < GM_ROWS) pairs_lds[threadIdx.x] = first + (int)threadIdx.x < plan[e + 1] ? plan[E + 1 + first + threadIdx.x] : -1;
-    __syncthreads();
+    for (int r = threadIdx.x; r < GM_ROWS; r += blockDim.x) pairs_lds[r] = first + r < plan[e + 1] ? plan[E + 1 + first + r] : -1;
     return e;
 }
 
-// act[pair][f] = bf16(silu(gate[e][f] . h[row]) * (up[e][f] . h[row])); a wave takes 32 pairs by 32 hidden units
-__global__ __launch_bounds__(256) void grouped_hidden_kernel(const bf16_t* __restrict__ h, const int32_t* __restrict__ plan, bf16_t* __restrict__ act,
-                                                             const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up, int E, int top, int D,
-                                                             int F) {
+// A workgroup of four waves takes GM_ROWS pairs of one expert by GM_COLS weight rows: K goes by in
+// steps of GM_BK columns that all threads stage in LDS, 16 bytes a thread and load (the pairs' rows
+// gathered), in rows padded by 16 bytes so that a fragment's 32 rows spread over the banks; a wave
+// takes 64 pairs by 32 weight rows.
+//   HIDDEN: the weight rows are GM_COLS hidden units of gate and of up, and
+//           out[pair][f] = bf16(silu(gate_f . h[pair / top]) * (up_f . h[pair / top]))
+//   else:   out[pair][d] = w0_d . a[pair], float
+#define GM_COLS 64
+#define GM_BK 64
+#define GM_LD (GM_BK + 8)
+template <bool HIDDEN>
+__global__ __launch_bounds__(256) void grouped_tile_kernel(const bf16_t* __restrict__ a, const int32_t* __restrict__ plan, void* __restrict__ out,
+                                                           const bf16_t* __restrict__ w0, const bf16_t* __restrict__ w1, int E, int top, int K,
+                                                           int N) {
+    constexpr int NB = HIDDEN ? 2 : 1;
     __shared__ int32_t pairs[GM_ROWS];
+    __shared__ __attribute__((aligned(16))) bf16_t As[GM_ROWS * GM_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[NB * GM_COLS * GM_LD];
     const int e = tile_of(plan, E, blockIdx.x, pairs);
     if (e < 0) return;
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, l32 = lane % 32, kq = lane / 32;
-    const int f0 = (blockIdx.y * 4 + wave) * 32;
-    if (f0 >= F) return;
-    const int my_pair = pairs[l32];
-    const bf16_t* a_row = h + (size_t)(my_pair >= 0 ? my_pair / top : 0) * D + kq * 8;
-    const size_t w_row = ((size_t)e * F + min(f0 + l32, F - 1)) * D + kq * 8;
-    const bf16_t* g_row = gate + w_row;
-    const bf16_t* u_row = up + w_row;
-    f32x16 acc_g, acc_u;
+    __syncthreads();
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, l32 = lane % 32, kq = lane / 32;
+    const int rh = wave / 2, uh = wave % 2, n0 = blockIdx.y * GM_COLS;
+    f32x16 acc[2][NB];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc_g[i] = acc_u[i] = 0.f;
-#pragma unroll 4
-    for (int k = 0; k < D; k += 16) {
-        const bf16x8 a = my_pair >= 0 ? load_chunk(a_row + k) : zero_chunk();
-        acc_g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(g_row + k), acc_g, 0, 0, 0);
-        acc_u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(u_row + k), acc_u, 0, 0, 0);
-    }
-    if (f0 + l32 >= F) return;
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int pair = pairs[8 * (i / 4) + i % 4 + 4 * kq];
-        if (pair >= 0) act[(size_t)pair * F + f0 + l32] = f32_to_bf16_bits(acc_g[i] / (1.f + expf(-acc_g[i])) * acc_u[i]);
-    }
-}
-
-// y[pair][d] = down[e][d] . act[pair]; a wave takes 32 pairs by 32 outputs
-__global__ __launch_bounds__(256) void grouped_down_kernel(const bf16_t* __restrict__ act, const int32_t* __restrict__ plan, float* __restrict__ y,
-                                                           const bf16_t* __restrict__ down, int E, int D, int F) {
-    __shared__ int32_t pairs[GM_ROWS];
-    const int e = tile_of(plan, E, blockIdx.x, pairs);
-    if (e < 0) return;
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, l32 = lane % 32, kq = lane / 32;
-    const int d0 = (blockIdx.y * 4 + wave) * 32;
-    if (d0 >= D) return;
-    const int my_pair = pairs[l32];
-    const bf16_t* a_row = act + (size_t)max(my_pair, 0) * F + kq * 8;
-    const bf16_t* w_row = down + ((size_t)e * D + min(d0 + l32, D - 1)) * F + kq * 8;
-    f32x16 acc;
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll 4
-    for (int k = 0; k < F; k += 16) {
-        const bf16x8 a = my_pair >= 0 ? load_chunk(a_row + k) : zero_chunk();
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, load_chunk(w_row + k), acc, 0, 0, 0);
-    }
-    if (d0 + l32 >= D) return;
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+    // what this thread stages at every step: chunk `ch` of four pairs' rows and of two (or four) weight rows
+    const int ch = tid % 8, r_first = tid / 8;              // rows r_first, r_first + 32, ...
+    const bf16_t* a_src[GM_ROWS / 32];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int pair = pairs[8 * (i / 4) + i % 4 + 4 * kq];
-        if (pair >= 0) y[(size_t)pair * D + d0 + l32] = acc[i];
+    for (int c = 0; c < GM_ROWS / 32; ++c) {
+        const int pair = pairs[r_first + 32 * c];
+        a_src[c] = pair >= 0 ? a + (size_t)(HIDDEN ? pair / top : pair) * K + ch * 8 : nullptr;
     }
+    const bf16_t* b_src[NB * GM_COLS / 32];
+#pragma unroll
+    for (int c = 0; c < NB * GM_COLS / 32; ++c) {
+        const int r = r_first + 32 * c;                     // rows GM_COLS and up are the second matrix's
+        const bf16_t* base = r < GM_COLS ? w0 : w1;
+        b_src[c] = base + ((size_t)e * N + min(n0 + r % GM_COLS, N - 1)) * K + ch * 8;
+    }
+    for (int k0 = 0; k0 < K; k0 += GM_BK) {
+        const bool inside = k0 + ch * 8 < K;                // (K is a multiple of 16, a chunk lies inside or outside)
+        bf16x8 av[GM_ROWS / 32], bv[NB * GM_COLS / 32];
+#pragma unroll
+        for (int c = 0; c < GM_ROWS / 32; ++c) av[c] = a_src[c] && inside ? load_chunk(a_src[c] + k0) : zero_chunk();
+#pragma unroll
+        for (int c = 0; c < NB * GM_COLS / 32; ++c) bv[c] = inside ? load_chunk(b_src[c] + k0) : zero_chunk();
+        __syncthreads();                                    // the step before has been read
+#pragma unroll
+        for (int c = 0; c < GM_ROWS / 32; ++c) *(bf16x8*)(As + (r_first + 32 * c) * GM_LD + ch * 8) = av[c];
+#pragma unroll
+        for (int c = 0; c < NB * GM_COLS / 32; ++c) *(bf16x8*)(Bs + (r_first + 32 * c) * GM_LD + ch * 8) = bv[c];
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < GM_BK / 16; ++ks) {
+            const int col = ks * 16 + kq * 8;
+            const bf16x8 a0 = *(const bf16x8*)(As + (rh * 64 + l32) * GM_LD + col);
+            const bf16x8 a1 = *(const bf16x8*)(As + (rh * 64 + 32 + l32) * GM_LD + col);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const bf16x8 bj = *(const bf16x8*)(Bs + (j * GM_COLS + uh * 32 + l32) * GM_LD + col);
+                acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, bj, acc[0][j], 0, 0, 0);
+                acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, bj, acc[1][j], 0, 0, 0);
+            }
+        }
+    }
+    const int n = n0 + uh * 32 + l32;
+    if (n >= N) return;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int pair = pairs[rh * 64 + i * 32 + 8 * (q / 4) + q % 4 + 4 * kq];
+            if (pair < 0) continue;
+            if constexpr (HIDDEN) {
+                const float g = acc[i][0][q];
+                ((bf16_t*)out)[(size_t)pair * N + n] = f32_to_bf16_bits(g / (1.f + expf(-g)) * acc[i][NB - 1][q]);
+            } else {
+                ((float*)out)[(size_t)pair * N + n] = acc[i][0][q];
+            }
+        }
 }
 
 // out[row] (+)= sum_k w[row][k] y[row][k], in the order of the picks
@@ -297,10 +334,11 @@ extern "C" int picolm_call_routed_experts(void* user, const picolm_step_view* v)
         moe_plan_kernel<<<1, 1024, sizeof(int32_t) * (2 * (size_t)E + 1), v->stream>>>(picks, plan, E, top, (int)n_pairs);
         PICOLM_LAUNCH_CHECK("routed_experts (plan)");
         const unsigned tiles = (unsigned)(ceil_div64(n_pairs, GM_ROWS) + E);      // no more than these are filled; the rest leave at once
-        grouped_hidden_kernel<<<dim3(tiles, ceil_div(F, 128)), 256, 0, v->stream>>>((const bf16_t*)v->in, plan, (bf16_t*)act, (const bf16_t*)a->gate,
-                                                                                   (const bf16_t*)a->up, E, top, D, F);
+        grouped_tile_kernel<true><<<dim3(tiles, ceil_div(F, GM_COLS)), 256, 0, v->stream>>>((const bf16_t*)v->in, plan, act, (const bf16_t*)a->gate,
+                                                                                           (const bf16_t*)a->up, E, top, D, F);
         PICOLM_LAUNCH_CHECK("routed_experts (hidden, grouped)");
-        grouped_down_kernel<<<dim3(tiles, ceil_div(D, 128)), 256, 0, v->stream>>>((const bf16_t*)act, plan, y, (const bf16_t*)a->down, E, D, F);
+        grouped_tile_kernel<false><<<dim3(tiles, ceil_div(D, GM_COLS)), 256, 0, v->stream>>>((const bf16_t*)act, plan, y, (const bf16_t*)a->down,
+                                                                                            nullptr, E, top, F, D);
         PICOLM_LAUNCH_CHECK("routed_experts (down, grouped)");
         grouped_sum_kernel<<<v->rows, 256, 0, v->stream>>>(y, picks, (float*)v->out, E, top, D, a->adds);
         PICOLM_LAUNCH_CHECK("routed_experts (sum)");

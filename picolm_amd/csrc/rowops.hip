@@ -168,16 +168,20 @@ extern "C" int picolm_call_slice_norm(void* user, const picolm_step_view* v) {
 }
 
 // ---- a product per head -----------------------------------------------------------------------------
-// One workgroup per (HL_ROWS rows, head): the rows' inputs wait in LDS as floats and every weight
-// that is read meets all of them.  Not transposed: a wave per output, its lanes along the input;
-// transposed: a thread per output, adjacent threads read adjacent weights.
+// One workgroup per (HL_ROWS rows, head, HL_COLS outputs): the rows' inputs wait in LDS as floats and
+// every weight that is read meets all of them.  Not transposed: a wave takes four outputs at a
+// time, its lanes along the input (adjacent lanes read adjacent weights).  Transposed: a thread per
+// output and quarter of the input, adjacent threads read adjacent weights, and the quarters meet in
+// LDS.  Either way a thread has several loads on their way at once: a decode step has few
+// workgroups, and what they wait for is the latency of their loads.
 #define HL_ROWS 8
+#define HL_COLS 64
 template <typename TW>
 __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_args a, const void* __restrict__ in, void* __restrict__ out,
                                                           const float* __restrict__ gate, int n_rows) {
-    extern __shared__ float hl_in[];      // [HL_ROWS][in_dim]
+    extern __shared__ float hl_in[];      // [HL_ROWS][in_dim] | partial sums [4][HL_ROWS][HL_COLS] (transposed)
     const int head = blockIdx.y, row0 = blockIdx.x * HL_ROWS, nr = min(HL_ROWS, n_rows - row0);
-    const int K = a.in_dim, N = a.out_dim;
+    const int K = a.in_dim, N = a.out_dim, o0 = blockIdx.z * HL_COLS;
     for (int idx = threadIdx.x; idx < HL_ROWS * K; idx += blockDim.x) {
         const int r = idx / K, i = idx % K;
         hl_in[idx] = r < nr ? load_as_f32(in, (size_t)(row0 + r) * a.in_stride + a.in_off + (size_t)head * K + i, a.in_dtype) : 0.f;
@@ -193,37 +197,58 @@ __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_arg
         store_from_f32(out, row * a.out_stride + a.out_off + (size_t)head * N + o, a.out_dtype, acc);
     };
     if (a.transposed) {
+        float* part = hl_in + HL_ROWS * K;
         const TW* wh = w + (size_t)head * K * N;
-        for (int o = threadIdx.x; o < N; o += blockDim.x) {
-            float acc[HL_ROWS];
+        const int col = threadIdx.x % HL_COLS, quarter = threadIdx.x / HL_COLS, o = o0 + col;
+        const int per = (K + 3) / 4, i0 = quarter * per, i1 = min(K, i0 + per);
+        float acc[HL_ROWS];
 #pragma unroll
-            for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
-            for (int i = 0; i < K; ++i) {
+        for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
+        if (o < N) {
+#pragma unroll 8
+            for (int i = i0; i < i1; ++i) {
                 const float wv = to_f32<TW>(wh[(size_t)i * N + o]);
 #pragma unroll
                 for (int r = 0; r < HL_ROWS; ++r) acc[r] += wv * hl_in[r * K + i];
             }
+        }
 #pragma unroll
-            for (int r = 0; r < HL_ROWS; ++r)
-                if (r < nr) finish(r, o, acc[r]);
+        for (int r = 0; r < HL_ROWS; ++r) part[(quarter * HL_ROWS + r) * HL_COLS + col] = acc[r];
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < HL_ROWS * HL_COLS; idx += blockDim.x) {
+            const int r = idx / HL_COLS, c = idx % HL_COLS;
+            if (r < nr && o0 + c < N)
+                finish(r, o0 + c, part[(0 * HL_ROWS + r) * HL_COLS + c] + part[(1 * HL_ROWS + r) * HL_COLS + c] +
+                                      part[(2 * HL_ROWS + r) * HL_COLS + c] + part[(3 * HL_ROWS + r) * HL_COLS + c]);
         }
     } else {
-        const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, n_waves = blockDim.x / WAVE;
+        const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
         const TW* wh = w + (size_t)head * N * K;
-        for (int o = wave; o < N; o += n_waves) {
-            float acc[HL_ROWS];
+        const int o_end = min(N, o0 + HL_COLS);
+        for (int ob = o0 + wave * 4; ob < o_end; ob += 16) {        // four waves, four outputs each at a time
+            float acc[4][HL_ROWS];
 #pragma unroll
-            for (int r = 0; r < HL_ROWS; ++r) acc[r] = 0.f;
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int r = 0; r < HL_ROWS; ++r) acc[u][r] = 0.f;
             for (int i = lane; i < K; i += WAVE) {
-                const float wv = to_f32<TW>(wh[(size_t)o * K + i]);
+                float wv[4];
 #pragma unroll
-                for (int r = 0; r < HL_ROWS; ++r) acc[r] += wv * hl_in[r * K + i];
+                for (int u = 0; u < 4; ++u) wv[u] = ob + u < o_end ? to_f32<TW>(wh[(size_t)(ob + u) * K + i]) : 0.f;
+#pragma unroll
+                for (int r = 0; r < HL_ROWS; ++r) {
+                    const float x = hl_in[r * K + i];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc[u][r] += wv[u] * x;
+                }
             }
 #pragma unroll
-            for (int r = 0; r < HL_ROWS; ++r) {
-                const float s = wave_sum(acc[r]);
-                if (lane == 0 && r < nr) finish(r, o, s);
-            }
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int r = 0; r < HL_ROWS; ++r) {
+                    const float s = wave_sum(acc[u][r]);
+                    if (lane == 0 && r < nr && ob + u < o_end) finish(r, ob + u, s);
+                }
         }
     }
 }
@@ -243,10 +268,11 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
     PICOLM_REQUIRE(!a->gate_act || (v->extra[0] && a->gate_off >= 0 && a->gate_off + (int64_t)a->heads * a->out_dim <= a->gate_stride &&
                                     v->extra_row_bytes[0] >= (int64_t)a->gate_stride * 4),
                    "head_linear: the gate's rows of %d floats do not hold the heads at %d", a->gate_stride, a->gate_off);
-    const size_t lds = sizeof(float) * HL_ROWS * (size_t)a->in_dim;
-    PICOLM_REQUIRE(lds <= 64 * 1024, "head_linear: an input of %d a head needs %zu bytes of LDS", a->in_dim, lds);
+    const size_t lds = sizeof(float) * (HL_ROWS * (size_t)a->in_dim + (a->transposed ? 4 * HL_ROWS * HL_COLS : 0));
+    PICOLM_REQUIRE(lds <= 64 * 1024 && ceil_div(a->out_dim, HL_COLS) <= 65535, "head_linear: an input of %d a head needs %zu bytes of LDS",
+                   a->in_dim, lds);
     if (v->rows <= 0) return 0;
-    const dim3 grid(ceil_div(v->rows, HL_ROWS), a->heads);
+    const dim3 grid(ceil_div(v->rows, HL_ROWS), a->heads, ceil_div(a->out_dim, HL_COLS));
     if (a->weight_dt == PICOLM_F32)
         head_linear_kernel<float><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);
     else
@@ -256,9 +282,10 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
 }
 
 // ---- the sum and the norm of a layer that norms after adding ---------------------------------------------
+template <typename T>
 __global__ __launch_bounds__(1024) void gated_postnorm_kernel(float* __restrict__ x, const float* __restrict__ u, const float* __restrict__ g,
                                                              const float* __restrict__ bias, const float* __restrict__ weight, int W,
-                                                             float alpha, float eps) {
+                                                             float alpha, float eps, T* __restrict__ plain) {
     __shared__ float scratch[16];
     const size_t row = blockIdx.x;
     float* xr = x + row * W;
@@ -276,18 +303,28 @@ __global__ __launch_bounds__(1024) void gated_postnorm_kernel(float* __restrict_
     }
     ssq = block_sum(ssq, scratch);
     const float inv = 1.f / sqrtf(ssq / (float)W + eps);
-    for (int c = threadIdx.x; c < W; c += blockDim.x) xr[c] = sum_at(c) * inv * weight[c];      // a thread writes what only it reads
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float y = sum_at(c) * inv * weight[c];
+        xr[c] = y;                                                 // a thread writes what only it reads
+        if (plain) plain[row * W + c] = from_f32<T>(y);
+    }
 }
 
 extern "C" int picolm_call_gated_postnorm(void* user, const picolm_step_view* v) {
     const picolm_gated_postnorm_args* a = (const picolm_gated_postnorm_args*)user;
     VIEW_REQUIRE("gated_postnorm", v);
     PICOLM_REQUIRE(a && a->weight && v->in && v->out && a->width > 0, "gated_postnorm: weights or buffers are missing");
-    PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * 4 && (!v->extra[0] || v->extra_row_bytes[0] >= a->width * 4),
+    PICOLM_REQUIRE(v->in_row_bytes >= a->width * 4 && v->out_row_bytes >= a->width * 4 && (!v->extra[0] || v->extra_row_bytes[0] >= a->width * 4) &&
+                       (!v->extra[1] || v->extra_row_bytes[1] >= a->width * elem_bytes(v->dtype)),
                    "gated_postnorm: rows too short for a width of %d", a->width);
     if (v->rows <= 0) return 0;
-    gated_postnorm_kernel<<<v->rows, a->width >= 2048 ? 1024 : 256, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0],
-                                                                                   a->gate_bias, a->weight, a->width, a->alpha, a->eps);
+    const int threads = a->width >= 2048 ? 1024 : 256;
+    if (v->dtype == PICOLM_F32)
+        gated_postnorm_kernel<float><<<v->rows, threads, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0], a->gate_bias,
+                                                                        a->weight, a->width, a->alpha, a->eps, (float*)v->extra[1]);
+    else
+        gated_postnorm_kernel<bf16_t><<<v->rows, threads, 0, v->stream>>>((float*)v->out, (const float*)v->in, (const float*)v->extra[0], a->gate_bias,
+                                                                         a->weight, a->width, a->alpha, a->eps, (bf16_t*)v->extra[1]);
     PICOLM_LAUNCH_CHECK("gated_postnorm");
     return 0;
 }

@@ -106,16 +106,19 @@ class PostNormBlock(Block):
             self.mu = fetch.get(self.shift_name).to(torch.float32).contiguous()
         self.gate_bias = [fetch.get(g.names[0] + ".b").to(torch.float32).contiguous() for g in self.gates]
 
-    def _join(self, b, x: int, branch: int, plain: int, which: int, norm) -> None:
-        """x <- norm(alpha x + branch * gate(plain))"""
+    def _join(self, b, x: int, branch: int, plain: int, which: int, norm, leaves_plain: bool = False) -> None:
+        """x <- norm(alpha x + branch * gate(plain)); leaves_plain: and the new x in `plain`, in the
+        dtype that products read."""
         import torch
         from .. import kernels
         from .calls import GatedPostnormArgs, emit_library_call
-        extra, bias = [], None
+        extra, bias = [-1], None
         if self.gates:
             g = b.buffer("postnorm.gate", self.D, torch.float32)
             self.gates[which].emit(b, plain, g, kernels.EPI_STORE)
             extra, bias = [g], self.gate_bias[which]
+        if leaves_plain:
+            extra.append(plain)
         ref = norm.norm_ref()
         if ref is None:
             raise ValueError("a block that norms after the sum takes RMS norms")
@@ -147,9 +150,8 @@ class PostNormBlock(Block):
             plain = reads = self._plain_rows(b, x)
         branch = b.buffer("postnorm.branch", D, torch.float32)
         self.inner.emit(b, Rows(reads), branch, accumulate=False)
-        self._join(b, x, branch, plain, 0, self.mixer_norm)
+        self._join(b, x, branch, plain, 0, self.mixer_norm, leaves_plain=self.ffn is not None)
         if self.ffn is not None:
-            plain = self._plain_rows(b, x)
             self.ffn.emit(b, Rows(plain), branch, accumulate=False)
             self._join(b, x, branch, plain, 1, self.ffn_norm)
 

@@ -27,7 +27,7 @@ def test_the_registry_knows_the_name_and_the_configuration_round_trips():
     (("layers", 3, "mixer", "kv_rank"), 2000, "layers[3].mixer.kv_rank"), (("layers", 3, "mixer", "scale"), None, "layers[3].mixer.scale"),
     (("layers", 0, "mlp", "kind"), "dense", "layers[0].mlp.kind"), (("layers", 0, "mlp", "router", "top"), 9, "layers[0].mlp.router.top"),
     (("layers", 3, "mlp", "shared"), 5, "layers[3].mlp.shared"), (("layers", 4, "weights_of"), 4, "layers[4].weights_of"),
-    (("layers", 4, "weights_of"), 1, "layers[4].weights_of"), (("layers", 5, "weights_of"), 0, "layers[5].weights_of"),
+    (("layers", 5, "weights_of"), 0, "layers[5].weights_of"), (("layers", 3, "mixer", "scale"), 0.0, "layers[3].mixer.scale"),
     (("layers", 1, "weights_of"), 7, "layers[1].weights_of"),
 ])
 def test_a_fault_names_its_key(path, value, names):
@@ -57,6 +57,18 @@ def test_layer_runs_share_blocks_and_keep_entries_of_their_own():
     assert sizes == {D, D + 3 * 24 * 20, D + 2 * 100 + 100 * 12}
     [group] = model.cache_spec.kv_groups
     assert (group.n_entries, group.n_kv_heads, group.head_dim) == (2, 1, 40)      # the latents are the keys, one head of them
+
+
+def test_a_layer_may_name_one_that_names_another():
+    cfg = copy.deepcopy(zt.CONFIG_A)
+    cfg["layers"][4]["weights_of"] = 4          # itself
+    with pytest.raises(ConfigError):
+        ZarinexConfig.from_dict(cfg)
+    cfg["layers"].append(copy.deepcopy(cfg["layers"][1]))
+    cfg["layers"][4]["weights_of"] = 0
+    cfg["layers"][6]["weights_of"] = 1          # which runs with layer 3's
+    model = build_from_config_dict(cfg)
+    assert [c.block for c in model.order] == [0, 2, 1, 2, 0, 1, 2]
 
 
 def test_the_plain_positions():
