@@ -20,6 +20,16 @@
 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+// e^x for x <= 0 through the hardware's 2^y, with the rounding of y = x log2(e) carried along:
+// y = hi + lo, e^x = 2^hi (1 + lo ln 2).  Within two units in the last place, at a tenth of the
+// library function's instructions; a walk takes it once per state element and token.
+__device__ __forceinline__ float exp_of_decay(float x) {
+    const float log2e_hi = 1.44269502162933349609375f, log2e_lo = 1.925963033500011e-8f;
+    const float hi = x * log2e_hi;
+    const float lo = fmaf(x, log2e_hi, -hi) + x * log2e_lo;
+    return __builtin_amdgcn_exp2f(hi) * fmaf(lo, 0.693147182464599609375f, 1.f);
+}
+
 #define DS_TB 16         // tokens whose q, k, decays and inputs wait in LDS at a time
 #define DS_KPT 16        // rows of the state a thread keeps in registers
 #define DS_MAX_KEY_DIM 256
@@ -47,11 +57,13 @@ __device__ __forceinline__ float* ds_ws(const DecayScan& a, int seq, int chunk, 
     return a.ws + ((((size_t)seq * a.chunks_per_seq + chunk) * a.heads + head) * 3 + part) * a.key_dim * a.value_dim;
 }
 
-template <int R>
+// KIND: 1 a decay per row, 2 exp(dt A) per element; TRACK: pass 1 of the chunked walk (no outputs, the decays' products kept)
+template <int R, int KIND, bool TRACK>
 __global__ __launch_bounds__(256) void decay_scan_kernel(DecayScan a) {
     extern __shared__ float ds_lds[];
     constexpr int CW = WAVE / R;
-    const int kpt = a.kpt, kd = kpt * R, CB = a.n_waves * CW;
+    constexpr int kpt = DS_KPT, kd = kpt * R;      // rows past key_dim are zeros that stay zeros: no test per row in the walk
+    const int CB = a.n_waves * CW;
     float* ks = ds_lds;                      // [TB][kd]
     float* qs = ks + DS_TB * kd;             // [TB][kd]
     float* as = qs + DS_TB * kd;             // [TB][kd]   (kind 1)
@@ -77,10 +89,10 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(DecayScan a) {
         const int kr = i * R + r;
         const bool in = i < kpt && valid && kr < a.key_dim;
         if (a.mode == 0) S[i] = in ? st[(size_t)kr * a.value_dim + j] : 0.f;
-        else if (a.mode == 1) S[i] = 0.f;
+        else if (TRACK) S[i] = 0.f;
         else S[i] = in ? ds_ws(a, seq, chunk, head, 2)[(size_t)kr * a.value_dim + j] : 0.f;
         P[i] = 1.f;
-        Ar[i] = in && a.kind == 2 ? a.A[channel * a.key_dim + kr] : 0.f;
+        Ar[i] = in && KIND == 2 ? a.A[channel * a.key_dim + kr] : 0.f;
     }
     const float skip = a.skip && valid ? a.skip[channel] : 0.f;
     for (int b0 = row0; b0 < row1; b0 += DS_TB) {
@@ -92,41 +104,40 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(DecayScan a) {
             const bool in = i < a.key_dim;
             ks[idx] = in ? src[a.k_off] : 0.f;
             qs[idx] = in ? src[a.q_off] : 0.f;
-            if (a.kind == 1) as[idx] = in ? src[a.a_off] : 0.f;
+            if (KIND == 1) as[idx] = in ? src[a.a_off] : 0.f;
         }
         for (int idx = tid; idx < nb * CB; idx += blockDim.x) {
             const int t = idx / CB, c = cb * CB + idx % CB;
             const bool in = c < a.value_dim;
             const size_t ch = (size_t)head * a.value_dim + c;
             xs[idx] = in ? a.x[(size_t)(b0 + t) * a.x_stride + a.x_off + ch] : 0.f;
-            if (a.kind == 2)
+            if (KIND == 2)
                 dts[idx] = in ? softplus_f(a.dt[(size_t)(b0 + t) * a.dt_stride + a.dt_off + ch] + (a.dt_bias ? a.dt_bias[ch] : 0.f)) : 0.f;
         }
         __syncthreads();
         for (int t = 0; t < nb; ++t) {
             const float xv = xs[t * CB + col];
-            const float dtv = a.kind == 2 ? dts[t * CB + col] : 1.f;
+            const float dtv = KIND == 2 ? dts[t * CB + col] : 1.f;
             const float wv = dtv * xv;
             const float* k = ks + t * kd + r;
             const float* q = qs + t * kd + r;
             const float* ar = as + t * kd + r;
             float o = 0.f;
 #pragma unroll
-            for (int i = 0; i < DS_KPT; ++i)
-                if (i < kpt) {
-                    const float decay = a.kind == 2 ? expf(dtv * Ar[i]) : ar[i * R];
-                    S[i] = decay * S[i] + k[i * R] * wv;
-                    if (a.mode == 1) P[i] *= decay;
-                    o += S[i] * q[i * R];
-                }
-            if (a.mode == 1) continue;
+            for (int i = 0; i < DS_KPT; ++i) {
+                const float decay = KIND == 2 ? exp_of_decay(dtv * Ar[i]) : ar[i * R];
+                S[i] = decay * S[i] + k[i * R] * wv;
+                if (TRACK) P[i] *= decay;
+                else o += S[i] * q[i * R];
+            }
+            if (TRACK) continue;
             for (int off = CW; off < WAVE; off <<= 1) o += __shfl_xor(o, off, WAVE);
             if (r == 0 && valid) a.out[(size_t)(b0 + t) * a.heads * a.value_dim + channel] = o + skip * xv;
         }
     }
     if (a.mode == 3) return;
     float* n_out = a.mode == 0 ? st : ds_ws(a, seq, chunk, head, 0);
-    float* p_out = a.mode == 1 ? ds_ws(a, seq, chunk, head, 1) : nullptr;
+    float* p_out = TRACK ? ds_ws(a, seq, chunk, head, 1) : nullptr;
 #pragma unroll
     for (int i = 0; i < DS_KPT; ++i) {
         const int kr = i * R + r;
@@ -212,7 +223,7 @@ extern "C" int picolm_call_decay_scan(void* user, const picolm_step_view* v) {
     int R = 1;
     while (R * DS_KPT < kd) R *= 2;
     s.R = R;
-    s.kpt = ceil_div(kd, R);
+    s.kpt = DS_KPT;
     s.mode = 0, s.chunk_len = 0, s.chunks_per_seq = 1, s.ws = nullptr;
     const int CW = WAVE / R;
     auto launch = [&](int units) -> int {
@@ -225,11 +236,19 @@ extern "C" int picolm_call_decay_scan(void* user, const picolm_step_view* v) {
         PICOLM_REQUIRE(blocks < (1ll << 31), "decay_scan: %lld workgroups exceed the grid", (long long)blocks);
         const size_t lds = sizeof(float) * DS_TB * ((size_t)3 * s.kpt * R + 2 * n_waves * CW);
         const dim3 grid((unsigned)blocks), block(n_waves * WAVE);
-        if (R == 1) decay_scan_kernel<1><<<grid, block, lds, v->stream>>>(s);
-        else if (R == 2) decay_scan_kernel<2><<<grid, block, lds, v->stream>>>(s);
-        else if (R == 4) decay_scan_kernel<4><<<grid, block, lds, v->stream>>>(s);
-        else if (R == 8) decay_scan_kernel<8><<<grid, block, lds, v->stream>>>(s);
-        else decay_scan_kernel<16><<<grid, block, lds, v->stream>>>(s);
+#define DS_LAUNCH(RR)                                                                                              \
+    do {                                                                                                          \
+        if (s.kind == 1 && s.mode == 1) decay_scan_kernel<RR, 1, true><<<grid, block, lds, v->stream>>>(s);       \
+        else if (s.kind == 1) decay_scan_kernel<RR, 1, false><<<grid, block, lds, v->stream>>>(s);                \
+        else if (s.mode == 1) decay_scan_kernel<RR, 2, true><<<grid, block, lds, v->stream>>>(s);                 \
+        else decay_scan_kernel<RR, 2, false><<<grid, block, lds, v->stream>>>(s);                                 \
+    } while (0)
+        if (R == 1) DS_LAUNCH(1);
+        else if (R == 2) DS_LAUNCH(2);
+        else if (R == 4) DS_LAUNCH(4);
+        else if (R == 8) DS_LAUNCH(8);
+        else DS_LAUNCH(16);
+#undef DS_LAUNCH
         PICOLM_LAUNCH_CHECK("decay_scan");
         return 0;
     };

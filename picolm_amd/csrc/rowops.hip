@@ -9,6 +9,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "gemm_mfma.h"
 
 #define VIEW_REQUIRE(who, v)                                                                                      \
     PICOLM_REQUIRE((v) && (v)->struct_bytes == (int32_t)sizeof(picolm_step_view), "%s: the step view is of another version", who)
@@ -253,6 +254,51 @@ __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_arg
     }
 }
 
+// The same on the matrix cores, for steps of many rows in bfloat16 (not transposed): a wave takes 32
+// rows by 32 outputs of a head with v_mfma_f32_32x32x16_bf16, its operands straight from global
+// memory (float inputs are rounded to bfloat16 on the way, as every product's input is).
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(picolm_head_linear_args a, const void* __restrict__ in, void* __restrict__ out,
+                                                               const float* __restrict__ gate, int n_rows) {
+    const int head = blockIdx.y, row0 = blockIdx.x * 32, K = a.in_dim, N = a.out_dim;
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, l32 = lane % 32, kq = lane / 32;
+    const int n0 = (blockIdx.z * 4 + wave) * 32;
+    if (n0 >= N) return;
+    const int my_row = row0 + l32;
+    const size_t in_at = (size_t)min(my_row, n_rows - 1) * a.in_stride + a.in_off + (size_t)head * K + kq * 8;
+    const bf16_t* w_row = (const bf16_t*)a.weight + ((size_t)head * N + min(n0 + l32, N - 1)) * K + kq * 8;
+    f32x16 acc;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) acc[q] = 0.f;
+#pragma unroll 4
+    for (int k = 0; k < K; k += 16) {
+        bf16x8 av;
+        if (a.in_dtype == PICOLM_F32) {
+            const float4 lo = *(const float4*)((const float*)in + in_at + k), hi = *(const float4*)((const float*)in + in_at + k + 4);
+            const float f[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            bf16_t* bits = (bf16_t*)&av;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) bits[i] = f32_to_bf16_bits(f[i]);
+        } else {
+            av = load_chunk((const bf16_t*)in + in_at + k);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, load_chunk(w_row + k), acc, 0, 0, 0);
+    }
+    const int o = n0 + l32;
+    if (o >= N) return;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+        const size_t row = row0 + 8 * (q / 4) + q % 4 + 4 * kq;
+        if (row >= (size_t)n_rows) continue;
+        float y = acc[q];
+        if (a.gate_act) {
+            const float z = gate[row * a.gate_stride + a.gate_off + (size_t)head * N + o];
+            y *= a.gate_act == 1 ? silu_f(z) : sigmoid_f(z);
+        }
+        store_from_f32(out, row * a.out_stride + a.out_off + (size_t)head * N + o, a.out_dtype, y);
+    }
+}
+#define HL_MFMA_FROM_ROWS 32
+
 extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
     const picolm_head_linear_args* a = (const picolm_head_linear_args*)user;
     VIEW_REQUIRE("head_linear", v);
@@ -272,6 +318,13 @@ extern "C" int picolm_call_head_linear(void* user, const picolm_step_view* v) {
     PICOLM_REQUIRE(lds <= 64 * 1024 && ceil_div(a->out_dim, HL_COLS) <= 65535, "head_linear: an input of %d a head needs %zu bytes of LDS",
                    a->in_dim, lds);
     if (v->rows <= 0) return 0;
+    if (v->dtype == PICOLM_BF16 && a->weight_dt == PICOLM_BF16 && !a->transposed && v->rows >= HL_MFMA_FROM_ROWS && a->in_dim % 16 == 0 &&
+        a->in_off % 8 == 0 && a->in_stride % 8 == 0 && ceil_div(a->out_dim, 128) <= 65535) {
+        head_linear_mfma_kernel<<<dim3(ceil_div(v->rows, 32), a->heads, ceil_div(a->out_dim, 128)), 256, 0, v->stream>>>(
+            *a, v->in, v->out, (const float*)v->extra[0], v->rows);
+        PICOLM_LAUNCH_CHECK("head_linear (matrix cores)");
+        return 0;
+    }
     const dim3 grid(ceil_div(v->rows, HL_ROWS), a->heads, ceil_div(a->out_dim, HL_COLS));
     if (a->weight_dt == PICOLM_F32)
         head_linear_kernel<float><<<grid, 256, lds, v->stream>>>(*a, v->in, v->out, (const float*)v->extra[0], v->rows);

@@ -35,6 +35,7 @@ class LatentAttention(Mixer):
         self.uq = Linear([prefix + "uq"], [n_heads * head_dim], q_rank)
         self.o = Linear([prefix + "o"], [hidden_size], n_heads * v_head_dim)
         self.uk = self.uv = self.q_norm = self.c_norm = None
+        self.uk_transposed = False
 
     def children(self):
         return [self.proj, self.uq, self.o]
@@ -47,6 +48,11 @@ class LatentAttention(Mixer):
     def load(self, fetch, runtime: Runtime) -> None:
         kept = lambda name: (lambda t: t.to(torch.float32) if runtime.is_f32 else t)(fetch.get(self.prefix + name)).contiguous()
         self.uk, self.uv = kept("uk"), kept("uv")
+        # the bfloat16 runtime keeps W_uk transposed per head, [heads][kv_rank][dim]: q' = W_uk^T q is then a plain product
+        # per head, which the matrix cores take; the 32-bit runtime multiplies with the tensor as it is stored
+        self.uk_transposed = not runtime.is_f32
+        if self.uk_transposed:
+            self.uk = self.uk.view(self.H, self.d, self.r).transpose(1, 2).contiguous().view(self.H * self.r, self.d)
         self.q_norm = fetch.get(self.prefix + "dq.norm").to(torch.float32).contiguous()
         self.c_norm = fetch.get(self.prefix + "dkv.norm").to(torch.float32).contiguous()
 
@@ -68,7 +74,8 @@ class LatentAttention(Mixer):
         # [W_uk^T q per head | c]: the attention's queries, and its one key and value
         qc = b.buffer("latent.qc", H * r + r, torch.float32)
         weight_dt = _DT[self.uk.dtype]
-        emit_library_call(b, "head_linear", HeadLinearArgs(b._ptr(self.uk), weight_dt, H, d, r, 1, H * d, 0, F32, H * r + r, 0, F32,
+        emit_library_call(b, "head_linear", HeadLinearArgs(b._ptr(self.uk), weight_dt, H, d, r, 0 if self.uk_transposed else 1, H * d, 0, F32,
+                                                           H * r + r, 0, F32,
                                                            GATE_NONE, 0, 0), qc, inp=q)
         emit_library_call(b, "slice_norm", SliceNormArgs(b._ptr(self.c_norm), r, width, rq, H * r + r, H * r, F32, self.eps), qc, inp=rows)
         scratch = b.buffer("latent.q.rows", H * r, b.dtype)
