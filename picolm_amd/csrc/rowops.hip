@@ -243,13 +243,16 @@ __global__ __launch_bounds__(256) void head_linear_kernel(picolm_head_linear_arg
                     for (int u = 0; u < 4; ++u) acc[u][r] += wv[u] * x;
                 }
             }
+            float mine = 0.f;                      // lane 8 u + r takes the sum of output u and row r: the gates are then loaded side by side
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
                 for (int r = 0; r < HL_ROWS; ++r) {
                     const float s = wave_sum(acc[u][r]);
-                    if (lane == 0 && r < nr && ob + u < o_end) finish(r, ob + u, s);
+                    if (lane == u * HL_ROWS + r) mine = s;
                 }
+            const int u = lane / HL_ROWS, r = lane % HL_ROWS;
+            if (lane < 4 * HL_ROWS && r < nr && ob + u < o_end) finish(r, ob + u, mine);
         }
     }
 }
