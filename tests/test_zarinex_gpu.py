@@ -81,6 +81,7 @@ ALONE = {
     "latent attention, latents of 64": one_layer(zt.latent(4, 24, 16, 64, 40, 0.3)),
     "latent attention, latents of 96, forty heads": one_layer(zt.latent(40, 8, 12, 96, 24, 0.5)),
     "latent attention, latents of 128": one_layer(zt.latent(2, 32, 48, 128, 64, 0.2)),
+    "latent attention, latents of 288": one_layer(zt.latent(2, 16, 24, 288, 48, 0.25)),      # beyond what a thread's registers hold of a key
     "latent attention, one head, latents of 5": one_layer(zt.latent(1, 7, 3, 5, 6, 0.6)),
     "forget-gated state": one_layer(zt.hgrn(3, 12, 20)),
     "forget-gated state, keys of 144": one_layer(zt.hgrn(2, 144, 8)),
